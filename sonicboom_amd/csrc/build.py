@@ -42,7 +42,8 @@ CORE_SOURCES = [
     "status.hip", "embed_norm.hip", "elementwise.hip", "gemm_plain.hip", "rope_kv.hip",
     "attention_plain.hip", "sampling.hip", "gemm_skinny.hip", "gemm_stream.hip", "gemm_mfma.hip",
     "random_fill.hip", "recurrent.hip", "attention_latent.hip", "attention_latent_mfma.hip",
-    "outnorm.hip", "headnorm_kv.hip", "moe.hip", "moe_mfma.hip",
+    "outnorm.hip", "headnorm_kv.hip", "moe.hip", "moe_mfma.hip", "timeconv.hip", "state_space.hip",
+    "attention_mixed.hip",
 ]
 HEADERS = ["common.h", "sb_hip.h", "mfma.h"]
 ATTN_SOURCES = ["attention_mfma.hip"]

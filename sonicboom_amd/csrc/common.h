@@ -47,6 +47,13 @@ __device__ __forceinline__ float swish_clamp_mul(float g, float u, float limit, 
   return (g / (1.0f + expf(-alpha * g))) * (u + 1.0f);
 }
 
+// The pair of an expert's gate and up products by the value of the experts' products' `gated` argument:
+// 1 the clamped swish pair above, 2 silu(g) u.
+__device__ __forceinline__ float expert_pair(float g, float u, int kind, float limit, float alpha) {
+  if (kind == 2) return (g / (1.0f + expf(-g))) * u;
+  return swish_clamp_mul(g, u, limit, alpha);
+}
+
 // The rotation of one pair (x0, x1) by the angle whose cosine and sine are c and s: every product
 // and sum rounded on its own (no fused multiply-add), so that every kernel that rotates a pair
 // gives the same bits (/root/reference/core/src/nn/rope.cpp:46-55).

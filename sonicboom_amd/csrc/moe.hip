@@ -20,15 +20,17 @@ constexpr int kMaxTop = 16;
 
 // One row's choice from its scores zr: the `top` largest in falling order (ties to the lower
 // number), the softmax over them, the gate.
+// score_kind 0: the weights are the softmax over the chosen z.  score_kind 1: the scores are sigmoid(z), the
+// largest scores are chosen and the weights are those scores times score_scale, not renormalized.
 __device__ __forceinline__ void route_row(int32_t *__restrict__ ids, float *__restrict__ weights, const float *zr, int r,
-                                          int n_experts, int top, int has_gate) {
+                                          int n_experts, int top, int has_gate, int score_kind = 0, float score_scale = 1.0f) {
   int chosen[kMaxTop];
   float score[kMaxTop];
   for (int k = 0; k < top; ++k) {
     int best = -1;
     float bz = 0.0f;
     for (int e = 0; e < n_experts; ++e) {
-      const float v = zr[e];
+      const float v = score_kind == 1 ? 1.0f / (1.0f + expf(-zr[e])) : zr[e];
       // candidates: below the last choice, or equal to it with a higher number (the order is
       // falling scores, rising numbers among equals); NaN scores are never chosen
       if (k > 0 && !(v < score[k - 1] || (v == score[k - 1] && e > chosen[k - 1]))) continue;
@@ -42,17 +44,17 @@ __device__ __forceinline__ void route_row(int32_t *__restrict__ ids, float *__re
   for (int k = 0; k < top; ++k) { w[k] = expf(score[k] - score[0]); sum += w[k]; }
   for (int k = 0; k < top; ++k) {
     ids[size_t(r) * top + k] = chosen[k];
-    weights[size_t(r) * (top + 1) + k] = w[k] / sum;
+    weights[size_t(r) * (top + 1) + k] = score_kind == 1 ? score[k] * score_scale : w[k] / sum;
   }
   weights[size_t(r) * (top + 1) + top] = has_gate ? 1.0f / (1.0f + expf(-zr[n_experts])) : 0.0f;
 }
 
 __global__ void __launch_bounds__(64)
 moe_route_kernel(int32_t *__restrict__ ids, float *__restrict__ weights, const float *__restrict__ z, int n_rows,
-                 int stride, int n_experts, int top, int has_gate) {
+                 int stride, int n_experts, int top, int has_gate, int score_kind, float score_scale) {
   const int r = blockIdx.x * 64 + threadIdx.x;
   if (r >= n_rows) return;
-  route_row(ids, weights, z + size_t(r) * stride, r, n_experts, top, has_gate);
+  route_row(ids, weights, z + size_t(r) * stride, r, n_experts, top, has_gate, score_kind, score_scale);
 }
 
 // The router's product and the choice in one launch: a block a row.  z_e = sum_k h[k] w[e][k] in
@@ -75,7 +77,8 @@ __device__ __forceinline__ void load8(const bf16_t *p, float (&v)[8]) {
 template <typename TX>
 __global__ void __launch_bounds__(256)
 moe_router_kernel(int32_t *__restrict__ ids, float *__restrict__ weights, const TX *__restrict__ h,
-                  const float *__restrict__ w, int n_rows, int n_in, int n_experts, int top, int has_gate) {
+                  const float *__restrict__ w, int n_rows, int n_in, int n_experts, int top, int has_gate, int score_kind,
+                  float score_scale) {
   extern __shared__ float zs[];                 // [n_z] scores, then [4][8] the waves' sums of a pass
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int r = blockIdx.x;
@@ -116,7 +119,7 @@ moe_router_kernel(int32_t *__restrict__ ids, float *__restrict__ weights, const 
     if (tid < 8 && e0 + tid < n_z) z[e0 + tid] = ((part[tid] + part[8 + tid]) + part[16 + tid]) + part[24 + tid];
     __syncthreads();
   }
-  if (tid == 0) route_row(ids, weights, z, r, n_experts, top, has_gate);
+  if (tid == 0) route_row(ids, weights, z, r, n_experts, top, has_gate, score_kind, score_scale);
 }
 
 template <typename TO>
@@ -150,7 +153,7 @@ moe_product_plain_kernel(TY *__restrict__ y, const TX *__restrict__ x, const TW 
     const TW *wu = wg + size_t(n_out) * n_in;
     float u = 0.0f;
     for (int k = 0; k < n_in; ++k) u = fmaf(xs[k], ld_f(wu, k), u);
-    g = swish_clamp_mul(g, u, limit, alpha);
+    g = expert_pair(g, u, gated, limit, alpha);
   }
   st_f(y, size_t(p) * n_out + o, g);
 }
@@ -159,20 +162,38 @@ moe_product_plain_kernel(TY *__restrict__ y, const TX *__restrict__ x, const TW 
 
 extern "C" int sb_moe_max_top(void) { return kMaxTop; }
 
+extern "C" int sb_moe_route_scored(int32_t *ids, float *weights, const float *z, int n_rows, int stride, int n_experts,
+                                   int top, int has_gate, int score_kind, float score_scale, void *stream);
 extern "C" int sb_moe_route(int32_t *ids, float *weights, const float *z, int n_rows, int stride, int n_experts,
                             int top, int has_gate, void *stream) {
+  return sb_moe_route_scored(ids, weights, z, n_rows, stride, n_experts, top, has_gate, 0, 1.0f, stream);
+}
+
+extern "C" int sb_moe_route_scored(int32_t *ids, float *weights, const float *z, int n_rows, int stride, int n_experts,
+                                   int top, int has_gate, int score_kind, float score_scale, void *stream) {
   SB_REQUIRE(ids && weights && z, "sb_moe_route: null pointer");
+  SB_REQUIRE(score_kind == 0 || score_kind == 1, "sb_moe_route: unknown kind of score %d", score_kind);
   SB_REQUIRE(n_rows >= 0 && n_experts > 0 && top > 0 && top <= n_experts && stride >= n_experts + (has_gate ? 1 : 0),
              "sb_moe_route: bad sizes rows=%d experts=%d top=%d stride=%d", n_rows, n_experts, top, stride);
   SB_SUPPORT(top <= kMaxTop, "sb_moe_route: %d choices a row are more than %d", top, kMaxTop);
   if (n_rows == 0) return SB_OK;
-  moe_route_kernel<<<(n_rows + 63) / 64, 64, 0, (hipStream_t)stream>>>(ids, weights, z, n_rows, stride, n_experts, top, has_gate);
+  moe_route_kernel<<<(n_rows + 63) / 64, 64, 0, (hipStream_t)stream>>>(ids, weights, z, n_rows, stride, n_experts, top, has_gate, score_kind, score_scale);
   return sb::check_launch("sb_moe_route");
 }
 
+extern "C" int sb_moe_router_scored(int32_t *ids, float *weights, const void *h, int h_dtype, const float *w, int n_rows,
+                                    int n_in, int n_experts, int top, int has_gate, int score_kind, float score_scale,
+                                    void *stream);
 extern "C" int sb_moe_router(int32_t *ids, float *weights, const void *h, int h_dtype, const float *w, int n_rows,
                              int n_in, int n_experts, int top, int has_gate, void *stream) {
+  return sb_moe_router_scored(ids, weights, h, h_dtype, w, n_rows, n_in, n_experts, top, has_gate, 0, 1.0f, stream);
+}
+
+extern "C" int sb_moe_router_scored(int32_t *ids, float *weights, const void *h, int h_dtype, const float *w, int n_rows,
+                                    int n_in, int n_experts, int top, int has_gate, int score_kind, float score_scale,
+                                    void *stream) {
   SB_REQUIRE(ids && weights && h && w, "sb_moe_router: null pointer");
+  SB_REQUIRE(score_kind == 0 || score_kind == 1, "sb_moe_router: unknown kind of score %d", score_kind);
   SB_REQUIRE(n_rows >= 0 && n_in > 0 && n_experts > 0 && top > 0 && top <= n_experts && sb::valid_dtype(h_dtype),
              "sb_moe_router: bad sizes rows=%d in=%d experts=%d top=%d", n_rows, n_in, n_experts, top);
   SB_SUPPORT(top <= kMaxTop && n_experts < 2048, "sb_moe_router: %d choices of %d experts are more than %d of 2047", top,
@@ -181,8 +202,8 @@ extern "C" int sb_moe_router(int32_t *ids, float *weights, const void *h, int h_
   hipStream_t s = (hipStream_t)stream;
   const size_t lds = size_t(n_experts + 1 + 32) * sizeof(float);
   const unsigned blocks = n_rows;
-  if (h_dtype == SB_F32) moe_router_kernel<float><<<blocks, 256, lds, s>>>(ids, weights, (const float *)h, w, n_rows, n_in, n_experts, top, has_gate);
-  else moe_router_kernel<bf16_t><<<blocks, 256, lds, s>>>(ids, weights, (const bf16_t *)h, w, n_rows, n_in, n_experts, top, has_gate);
+  if (h_dtype == SB_F32) moe_router_kernel<float><<<blocks, 256, lds, s>>>(ids, weights, (const float *)h, w, n_rows, n_in, n_experts, top, has_gate, score_kind, score_scale);
+  else moe_router_kernel<bf16_t><<<blocks, 256, lds, s>>>(ids, weights, (const bf16_t *)h, w, n_rows, n_in, n_experts, top, has_gate, score_kind, score_scale);
   return sb::check_launch("sb_moe_router");
 }
 

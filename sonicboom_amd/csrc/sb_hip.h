@@ -301,6 +301,68 @@ int sb_moe_product_bf16(void *y, int y_dtype, const void *x, const void *w, cons
 int sb_swish_clamp_mul(void *out, int out_dtype, const float *gu, int n_rows, int width, float limit, float alpha,
                        void *stream);
 
+/* The router with another kind of score: score_kind 0 as sb_moe_route / sb_moe_router; 1: the scores are
+ * sigmoid(z), the `top` largest are chosen and their weights are those scores times score_scale (not
+ * renormalized).  The experts' products take gated = 2 for the pair silu(g) u. */
+int sb_moe_route_scored(int32_t *ids, float *weights, const float *z, int n_rows, int stride, int n_experts,
+                        int top, int has_gate, int score_kind, float score_scale, void *stream);
+int sb_moe_router_scored(int32_t *ids, float *weights, const void *h, int h_dtype, const float *w, int n_rows,
+                         int n_in, int n_experts, int top, int has_gate, int score_kind, float score_scale,
+                         void *stream);
+
+/* A short causal convolution over time, channel by channel, over the rows of a step:
+ *   y[t,c] = act(sum_j w[c,j] in[t - taps + 1 + j, c] (+ bias[c])) (+ in[t,c] with residual)
+ * act 0 none, 1 SiLU.  The inputs before a step's first row are the sequence's state, f32
+ * [slots][taps - 1][channels], the last taps - 1 inputs of the steps before (zeros for a new sequence);
+ * sb_time_conv_keep moves it on after the rows have been computed, or sb_time_conv itself with keep = 1
+ * when every sequence brings one row.  in/out may be column ranges of wider rows (strides in elements). */
+int sb_time_conv_max_taps(void);
+int sb_time_conv(void *out, int out_dtype, int out_stride, const void *in, int in_dtype, int in_stride, const void *w,
+                 int w_dtype, const void *bias, int bias_dtype, float *state, const int32_t *row_seq,
+                 const int32_t *cu_rows, const int32_t *slots, int n_rows, int n_seqs, int channels, int taps, int act,
+                 int residual, int keep, void *stream);
+int sb_time_conv_keep(const void *in, int in_dtype, int in_stride, float *state, const int32_t *cu_rows,
+                      const int32_t *slots, int n_rows, int n_seqs, int channels, int taps, void *stream);
+
+/* Recurrences with a float32 matrix per head and sequence (state[slots[s]]), walked row by row.
+ * sb_ssd_scan: dt = softplus(dt_raw + dt_bias[a]); S = exp(-exp(a_log[a]) dt) S + dt B x^T (S is N x P);
+ *   out = (S^T C + d_skip[a] x) silu(z); head a reads B, C of group a / (heads / groups); C lies c_off
+ *   floats after B in a row of bc.
+ * sb_delta_scan: q, k (of head a / (heads / kv_heads)) to unit vectors (eps_unit inside the root), q times
+ *   D^-1/2; beta = sigmoid(b); g = exp(-exp(a_log[a]) softplus(decay + dt_bias)) per key channel;
+ *   S = g S; u = beta (v - S^T k); S += k u^T; o = S^T q; out = o / sqrt(mean(o^2) + eps) w sigmoid(gate).
+ *   qkv rows hold q [kv_heads D] | k [kv_heads D] | v [heads E]. */
+int sb_state_scan_max_rows(void);
+int sb_state_scan_max_cols(void);
+int sb_ssd_scan(float *out, int out_stride, const float *z, int z_stride, const float *x, int x_stride, const float *bc,
+                int bc_stride, int c_off, const float *dt, int dt_stride, const float *dt_bias, const float *a_log,
+                const float *d_skip, float *state, const int32_t *cu_rows, const int32_t *slots, int n_seqs, int heads,
+                int groups, int N, int P, void *stream);
+int sb_delta_scan(void *out, int out_dtype, int out_stride, const float *qkv, int qkv_stride, const float *beta,
+                  int beta_stride, const float *decay, int decay_stride, const float *gate, int gate_stride,
+                  const float *dt_bias, const float *a_log, const void *w, int w_dtype, float *state,
+                  const int32_t *cu_rows, const int32_t *slots, int n_seqs, int heads, int kv_heads, int D, int E,
+                  float eps, float eps_unit, void *stream);
+
+/* Attention whose heads share their weights.
+ * sb_qk_rownorm_store: from f32 rows [q: heads_q dk | k: heads_kv dk]: q / rms(q, the whole part) * q_w *
+ *   (1 + temp_coef ln(floor((p + 1) / temp_every) + 1)) out in q_dtype; with store, k / rms(k) * k_w into the
+ *   key cache at the row's position and, with values_from_keys, k as it came into the value cache.
+ * sb_attention_shared: O[row][g][c][:] = sum_j P_g(row, j) V_c(j), P_g the causal softmax of
+ *   scale q_g . k_kv(g)(j) - r1[g] ln(1 + r2[g] (p - j)) (r1, r2 NULL: no bias); out f32.
+ * sb_head_mix: out[row][h][:] = sum_g mix[h][g] O[row][g][kv(h)][:] (mix NULL: the identity). */
+int sb_qk_rownorm_store(void *q_out, int q_dtype, const float *qk, int row_stride, const void *q_w, const void *k_w,
+                        int w_dtype, float eps, float temp_coef, int temp_every, const int32_t *row_pos,
+                        const int32_t *row_seq, const int32_t *page_table, int max_pages, int n_pages, void *k_cache,
+                        void *v_cache, int cache_dtype, int n_rows, int heads_q, int heads_kv, int dk, int store,
+                        int values_from_keys, void *stream);
+int sb_attention_shared(float *out, const void *q, int act_dtype, const void *k_cache, const void *v_cache,
+                        int cache_dtype, const int32_t *page_table, int max_pages, int n_pages_total,
+                        const int32_t *row_pos, const int32_t *row_seq, int n_rows, int heads_q, int heads_kv,
+                        int head_dim, int v_dim, float scale, const float *r1, const float *r2, void *stream);
+int sb_head_mix(void *out, int out_dtype, const float *o, const void *mix, int mix_dtype, int n_rows, int heads_q,
+                int heads_kv, int v_dim, void *stream);
+
 /* ids[r] = index of the first maximum of logits[r,:].  Two stages over
  * sb_argmax_parts(vocab) parts of a row; part_val / part_idx hold n_rows * parts
  * partial results (NULL allowed when parts == 1). */

@@ -30,6 +30,9 @@ class LayerBinding:
     v_cache: Optional[torch.Tensor]
     writes_cache: bool
     state: Optional[torch.Tensor]    # [max_slots, *shape] or None
+    # per-sequence states by name, each [max_slots, *shape]: those of a mixer that keeps several
+    # (its state_spec() gives a dict), and under "block.<name>" those the block itself keeps
+    states: Optional[Dict[str, torch.Tensor]] = None
 
 
 class DecoderModel:
@@ -83,8 +86,14 @@ class DecoderModel:
                     need = need[:2] + (0 if 0 in (have[2], need[2]) else max(have[2], need[2]),) + need[3:]
                 self.cache_specs[e.cache] = need
             ss = mixer.state_spec()
-            if ss is not None:
+            if isinstance(ss, dict):
+                for name, one in ss.items():
+                    self.state_specs[(i, name)] = (tuple(one.shape), one.dtype)
+            elif ss is not None:
                 self.state_specs[i] = (tuple(ss.shape), ss.dtype)
+            own = getattr(self.blocks[e.block], "state_specs", None)
+            for name, one in (own() if own is not None else {}).items():
+                self.state_specs[(i, "block." + name)] = (tuple(one.shape), one.dtype)
         self.groups: List[GroupSpec] = group_entries(self.cache_specs)
 
     # ---- construction --------------------------------------------------------
@@ -125,5 +134,6 @@ class DecoderModel:
             k = v = g = None
             if e.cache is not None:
                 k, v, g = cache.entry_views(e.cache)
-            out.append(LayerBinding(i, g, k, v, e.writes_cache and e.cache is not None, cache.state.get(i)))
+            named = {key[1]: t for key, t in cache.state.items() if isinstance(key, tuple) and key[0] == i}
+            out.append(LayerBinding(i, g, k, v, e.writes_cache and e.cache is not None, cache.state.get(i), named or None))
         return out

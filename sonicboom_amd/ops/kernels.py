@@ -1288,14 +1288,14 @@ def moe_plan(ids: Optional[torch.Tensor], n_experts: int, n_pairs: Optional[int]
 
 
 def moe_product(x: torch.Tensor, w: MoEWeight, plan: MoEPlan, x_div: int, out_dtype: torch.dtype,
-                limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
-    """Y[p] = X[p // x_div] W_e^T for every pair p of ``plan``; a gated weight gives the clamped
-    swish pair of its two halves.  bfloat16 operands with an inner size in eights run on the matrix
+                limit: float = 0.0, alpha: float = 1.0, pair: str = "swish_clamp") -> torch.Tensor:
+    """Y[p] = X[p // x_div] W_e^T for every pair p of ``plan``; a gated weight gives the pair of its
+    two halves that ``pair`` names (the clamped swish pair, or "silu": silu(g) u).  bfloat16 operands with an inner size in eights run on the matrix
     cores, the pairs grouped by expert on the device; everything else takes the plain kernel."""
     if w.experts != plan.n_experts:
         raise KernelLibraryError(f"the plan counts {plan.n_experts} experts, the weight has {w.experts}")
     if not (w.fast and x.dtype == torch.bfloat16 and w.w.dtype == torch.bfloat16 and w.n_in % 8 == 0):
-        return moe_product_plain(x, w.w, plan.ids, plan.n_pairs, x_div, out_dtype, w.gated, limit, alpha)
+        return moe_product_plain(x, w.w, plan.ids, plan.n_pairs, x_div, out_dtype, w.gated, limit, alpha, pair)
     _dev(x)
     if x.dim() != 2 or x.shape[1] != w.n_in or (plan.n_pairs + x_div - 1) // x_div > x.shape[0]:
         raise KernelLibraryError(f"expert product shapes do not match: x {tuple(x.shape)}, w {tuple(w.w.shape)}, "
@@ -1304,7 +1304,7 @@ def moe_product(x: torch.Tensor, w: MoEWeight, plan: MoEPlan, x_div: int, out_dt
     y = torch.empty((plan.n_pairs, w.n_out), dtype=out_dtype, device=x.device)
     check(library.core().sb_moe_product_bf16(
         _p(y), _dt(y), _p(x), _p(w.w), _p(plan.order), _p(plan.tiles), _p(plan.n_tiles), plan.max_tiles, plan.tile_rows,
-        plan.n_pairs, int(x_div), w.n_out, w.n_in, 1 if w.gated else 0, float(limit), float(alpha), _stream()))
+        plan.n_pairs, int(x_div), w.n_out, w.n_in, EXPERT_PAIRS[pair] if w.gated else 0, float(limit), float(alpha), _stream()))
     return y
 
 
@@ -1373,22 +1373,25 @@ def moe_max_top() -> int:
     return int(library.core().sb_moe_max_top())
 
 
-def moe_route(z: torch.Tensor, n_experts: int, top: int, has_gate: bool):
+def moe_route(z: torch.Tensor, n_experts: int, top: int, has_gate: bool, score: str = "softmax_chosen", score_scale: float = 1.0):
     """From router scores ``z`` float32 [n, >= n_experts (+ 1)]: the ``top`` largest of the first
     ``n_experts`` of every row (ties to the lower number) as int32 [n, top], and float32 [n, top + 1]:
-    the softmax over the chosen scores, then sigmoid(z[:, n_experts]) with ``has_gate`` (else 0)."""
+    the softmax over the chosen scores, then sigmoid(z[:, n_experts]) with ``has_gate`` (else 0).
+    ``score`` "sigmoid": the scores are sigmoid(z), the largest are chosen and their weights are those
+    scores times ``score_scale``, not renormalized."""
     _dev(z)
     if z.dtype != torch.float32 or z.dim() != 2:
         raise KernelLibraryError("router scores must be float32 [rows, experts]")
     n = z.shape[0]
     ids = torch.empty((n, top), dtype=torch.int32, device=z.device)
     weights = torch.empty((n, top + 1), dtype=torch.float32, device=z.device)
-    check(library.core().sb_moe_route(_p(ids), _p(weights), _p(z), n, z.shape[1], int(n_experts), int(top),
-                                      1 if has_gate else 0, _stream()))
+    check(library.core().sb_moe_route_scored(_p(ids), _p(weights), _p(z), n, z.shape[1], int(n_experts), int(top),
+                                             1 if has_gate else 0, ROUTER_SCORES[score], float(score_scale), _stream()))
     return ids, weights
 
 
-def moe_router(h: torch.Tensor, w: torch.Tensor, n_experts: int, top: int, has_gate: bool):
+def moe_router(h: torch.Tensor, w: torch.Tensor, n_experts: int, top: int, has_gate: bool, score: str = "softmax_chosen",
+               score_scale: float = 1.0):
     """The router in one launch: z = h w^T in float32 (``w`` float32 [n_experts (+ 1 with
     ``has_gate``), width], ``h`` rows of either type), then what :func:`moe_route` gives."""
     _dev(h, w)
@@ -1398,8 +1401,8 @@ def moe_router(h: torch.Tensor, w: torch.Tensor, n_experts: int, top: int, has_g
     n = h.shape[0]
     ids = torch.empty((n, top), dtype=torch.int32, device=h.device)
     weights = torch.empty((n, top + 1), dtype=torch.float32, device=h.device)
-    check(library.core().sb_moe_router(_p(ids), _p(weights), _p(h), _dt(h), _p(w), n, h.shape[1], int(n_experts), int(top),
-                                       1 if has_gate else 0, _stream()))
+    check(library.core().sb_moe_router_scored(_p(ids), _p(weights), _p(h), _dt(h), _p(w), n, h.shape[1], int(n_experts),
+                                              int(top), 1 if has_gate else 0, ROUTER_SCORES[score], float(score_scale), _stream()))
     return ids, weights
 
 
@@ -1415,7 +1418,8 @@ def swish_clamp_mul(gu: torch.Tensor, out_dtype: torch.dtype, limit: float, alph
 
 
 def moe_product_plain(x: torch.Tensor, w: torch.Tensor, ids: Optional[torch.Tensor], n_pairs: int, x_div: int,
-                      out_dtype: torch.dtype, gated: bool = False, limit: float = 0.0, alpha: float = 1.0) -> torch.Tensor:
+                      out_dtype: torch.dtype, gated: bool = False, limit: float = 0.0, alpha: float = 1.0,
+                      pair: str = "swish_clamp") -> torch.Tensor:
     """Y[p] = X[p // x_div] W_e^T, e = ids[p] (None: expert 0), by the plain kernel.  ``w``
     [experts, out (or 2*out, gate over up, with ``gated``), in]; gated: the clamped swish pair
     g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit), u' = u cut to +-limit."""
@@ -1430,5 +1434,209 @@ def moe_product_plain(x: torch.Tensor, w: torch.Tensor, ids: Optional[torch.Tens
         raise KernelLibraryError("more pairs than rows to take them from")
     y = torch.empty((n_pairs, n_out), dtype=out_dtype, device=x.device)
     check(library.core().sb_moe_product(_p(y), _dt(y), _p(x), _dt(x), _p(w), _dt(w), _p(ids), n_pairs, int(x_div),
-                                        n_out, n_in, n_experts, 1 if gated else 0, float(limit), float(alpha), _stream()))
+                                        n_out, n_in, n_experts, EXPERT_PAIRS[pair] if gated else 0, float(limit), float(alpha), _stream()))
     return y
+
+
+# ---- short convolutions over time, recurrences with a matrix state, attention with shared weights ----
+ROUTER_SCORES = {"softmax_chosen": 0, "sigmoid": 1}      # score_kind of sb_moe_route_scored
+EXPERT_PAIRS = {"swish_clamp": 1, "silu": 2}             # `gated` of the experts' products
+
+
+def time_conv_max_taps() -> int:
+    return int(library.core().sb_time_conv_max_taps())
+
+
+def time_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor, ctx,
+              out_dtype: torch.dtype, activation: Optional[str] = None, residual: bool = False,
+              columns: Optional[tuple] = None) -> torch.Tensor:
+    """y[t] = act(sum_j weight[:, j] x[t - taps + 1 + j] (+ bias)) (+ x[t] with ``residual``), channel by
+    channel over the rows of every sequence of the step ``ctx``; the rows before a step's first are
+    the sequence's ``state`` float32 [slots, taps - 1, channels], which is moved on.  ``columns``
+    (first, count): the channels are that range of the columns of ``x``.  ``activation``: None or "silu"."""
+    _dev(x, weight, bias, state)
+    if x.dim() != 2 or weight.dim() != 2:
+        raise KernelLibraryError("the convolution takes rows [n, columns] and taps [channels, taps]")
+    first, channels = columns if columns is not None else (0, x.shape[1])
+    taps = weight.shape[1]
+    if weight.shape[0] != channels or first < 0 or first + channels > x.shape[1]:
+        raise KernelLibraryError(f"taps {tuple(weight.shape)} do not fit {channels} channels from column {first} of {x.shape[1]}")
+    if bias is not None and bias.numel() != channels:
+        raise KernelLibraryError(f"the bias has {bias.numel()} elements for {channels} channels")
+    if state.dtype != torch.float32 or state.dim() != 3 or tuple(state.shape[1:]) != (taps - 1, channels):
+        raise KernelLibraryError(f"the state must be float32 [slots, {taps - 1}, {channels}], not {tuple(state.shape)}")
+    if activation not in (None, "silu"):
+        raise KernelLibraryError(f"the convolution's activation is None or 'silu', not {activation!r}")
+    n = x.shape[0]
+    if n != ctx.n_rows:
+        raise KernelLibraryError("the rows are not those of the step")
+    _i32(ctx.row_seq, n, "row sequences")
+    _i32(ctx.cu_rows, ctx.n_seqs + 1, "first rows")
+    _i32(ctx.slots, ctx.n_seqs, "slots")
+    y = torch.empty((n, channels), dtype=out_dtype, device=x.device)
+    esize = x.element_size()
+    src = x.data_ptr() + first * esize
+    keep = 1 if n == ctx.n_seqs else 0
+    lib = library.core()
+    check(lib.sb_time_conv(_p(y), _dt(y), channels, src, _dt(x), x.shape[1], _p(weight), _dt(weight), _p(bias),
+                           _dt(bias) if bias is not None else 0, _p(state), _p(ctx.row_seq), _p(ctx.cu_rows), _p(ctx.slots),
+                           n, ctx.n_seqs, channels, taps, 1 if activation == "silu" else 0, 1 if residual else 0, keep, _stream()))
+    if not keep:
+        check(lib.sb_time_conv_keep(src, _dt(x), x.shape[1], _p(state), _p(ctx.cu_rows), _p(ctx.slots), n, ctx.n_seqs,
+                                    channels, taps, _stream()))
+    return y
+
+
+def _f32_vec(t: torch.Tensor, n: int, what: str) -> None:
+    if t.dtype != torch.float32 or t.numel() != n or not t.is_cuda or not t.is_contiguous():
+        raise KernelLibraryError(f"{what} must be {n} float32 numbers on the GPU")
+
+
+def _f32_rows(t: torch.Tensor, n: int, width: int, what: str) -> None:
+    """``t`` float32 [n, >= width] whose rows are contiguous (a column range of wider rows is fine)."""
+    if t.dtype != torch.float32 or t.dim() != 2 or t.shape[0] != n or t.shape[1] < width or t.stride(1) != 1 or not t.is_cuda:
+        raise KernelLibraryError(f"{what} must be float32 rows [{n}, {width}] on the GPU, not {tuple(t.shape)}")
+
+
+def state_scan_limits():
+    lib = library.core()
+    return int(lib.sb_state_scan_max_rows()), int(lib.sb_state_scan_max_cols())
+
+
+def ssd_scan(z: torch.Tensor, x: torch.Tensor, b: torch.Tensor, c: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor,
+             a_log: torch.Tensor, d_skip: torch.Tensor, state: torch.Tensor, ctx, heads: int, groups: int, n_state: int,
+             v_dim: int) -> torch.Tensor:
+    """The selective state-space recurrence over the rows of the step (see csrc/state_space.hip):
+    ``z``, ``x`` [n, heads * v_dim], ``b``, ``c`` [n, groups * n_state] (column ranges of one tensor),
+    ``dt`` [n, heads] before bias and softplus, all float32 (views of wider rows allowed);
+    ``state`` float32 [slots, heads, n_state, v_dim], moved on.  Returns y * silu(z), float32 [n, heads * v_dim]."""
+    n = ctx.n_rows
+    inner = heads * v_dim
+    _f32_rows(z, n, inner, "z")
+    _f32_rows(x, n, inner, "x")
+    _f32_rows(b, n, groups * n_state, "B")
+    _f32_rows(c, n, groups * n_state, "C")
+    _f32_rows(dt, n, heads, "dt")
+    if b.stride(0) != c.stride(0) or b.untyped_storage().data_ptr() != c.untyped_storage().data_ptr():
+        raise KernelLibraryError("B and C must be column ranges of the same rows")
+    for t, what in ((dt_bias, "dt_bias"), (a_log, "A_log"), (d_skip, "D")):
+        _f32_vec(t, heads, what)
+    if state.dtype != torch.float32 or tuple(state.shape[1:]) != (heads, n_state, v_dim) or not state.is_contiguous():
+        raise KernelLibraryError(f"the state must be float32 [slots, {heads}, {n_state}, {v_dim}]")
+    out = torch.empty((n, inner), dtype=torch.float32, device=z.device)
+    c_off = (c.data_ptr() - b.data_ptr()) // 4
+    check(library.core().sb_ssd_scan(_p(out), inner, _p(z), z.stride(0), _p(x), x.stride(0), _p(b), b.stride(0), c_off,
+                                     _p(dt), dt.stride(0), _p(dt_bias), _p(a_log), _p(d_skip), _p(state), _p(ctx.cu_rows),
+                                     _p(ctx.slots), ctx.n_seqs, heads, groups, n_state, v_dim, _stream()))
+    return out
+
+
+def delta_scan(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, gate: torch.Tensor, dt_bias: torch.Tensor,
+               a_log: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, ctx, heads: int, kv_heads: int, dim: int,
+               v_dim: int, eps: float, eps_unit: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """The delta rule with a decay per key channel over the rows of the step (see csrc/state_space.hip):
+    ``qkv`` [n, 2 * kv_heads * dim + heads * v_dim] after the short convolution, ``beta`` [n, heads],
+    ``decay`` [n, heads * dim], ``gate`` [n, heads * v_dim] before their activations, all float32;
+    ``state`` float32 [slots, heads, dim, v_dim], moved on.  Returns the normed, gated heads
+    [n, heads * v_dim] in ``out_dtype``."""
+    n = ctx.n_rows
+    _f32_rows(qkv, n, 2 * kv_heads * dim + heads * v_dim, "q, k and v")
+    _f32_rows(beta, n, heads, "beta")
+    _f32_rows(decay, n, heads * dim, "the decays")
+    _f32_rows(gate, n, heads * v_dim, "the gate")
+    _f32_vec(dt_bias, heads * dim, "dt_bias")
+    _f32_vec(a_log, heads, "A_log")
+    _dev(weight)
+    if weight.numel() != v_dim:
+        raise KernelLibraryError(f"the norm's weight has {weight.numel()} elements for values of {v_dim}")
+    if state.dtype != torch.float32 or tuple(state.shape[1:]) != (heads, dim, v_dim) or not state.is_contiguous():
+        raise KernelLibraryError(f"the state must be float32 [slots, {heads}, {dim}, {v_dim}]")
+    out = torch.empty((n, heads * v_dim), dtype=out_dtype, device=qkv.device)
+    check(library.core().sb_delta_scan(_p(out), _dt(out), heads * v_dim, _p(qkv), qkv.stride(0), _p(beta), beta.stride(0),
+                                       _p(decay), decay.stride(0), _p(gate), gate.stride(0), _p(dt_bias), _p(a_log),
+                                       _p(weight), _dt(weight), _p(state), _p(ctx.cu_rows), _p(ctx.slots), ctx.n_seqs, heads,
+                                       kv_heads, dim, v_dim, float(eps), float(eps_unit), _stream()))
+    return out
+
+
+def qk_rownorm_store(qk: torch.Tensor, q_dtype: torch.dtype, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
+                     eps: float, temp_coef: float, temp_every: int, row_pos: torch.Tensor, row_seq: torch.Tensor,
+                     k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], page_table: Optional[torch.Tensor],
+                     heads_q: int, heads_kv: int, head_dim: int, store: bool = True, values_from_keys: bool = True) -> torch.Tensor:
+    """Queries and keys normed over their whole projections (see csrc/attention_mixed.hip): from float32
+    rows [q | k] the queries in ``q_dtype``, times the temperature of the row's position; with ``store``
+    the normed keys into the key cache and, with ``values_from_keys``, the keys as they came into the
+    value cache."""
+    _dev(qk, q_weight, k_weight, row_pos, row_seq, k_cache, v_cache, page_table)
+    n = qk.shape[0]
+    qw, kw = heads_q * head_dim, heads_kv * head_dim
+    if qk.dtype != torch.float32 or qk.dim() != 2 or qk.shape[1] < qw + (kw if store else 0):
+        raise KernelLibraryError(f"the projections must be float32 [rows, {qw + (kw if store else 0)}]")
+    for w, m, what in ((q_weight, qw, "query"), (k_weight, kw, "key")):
+        if w is not None and (w.numel() != m or (q_weight is not None and w.dtype != q_weight.dtype)):
+            raise KernelLibraryError(f"the {what} norm's weight must have {m} elements (and both one type)")
+    _i32(row_pos, n, "row positions")
+    max_pages = n_pages = cache_dt = 0
+    if store:
+        _check_cache_kv(k_cache, v_cache, heads_kv, head_dim, head_dim)
+        _check_rows(row_pos, row_seq, page_table, n)
+        max_pages, n_pages, cache_dt = page_table.shape[1], k_cache.shape[0], _dt(k_cache)
+    q = torch.empty((n, qw), dtype=q_dtype, device=qk.device)
+    wt = q_weight if q_weight is not None else k_weight
+    check(library.core().sb_qk_rownorm_store(
+        _p(q), _dt(q), _p(qk), qk.shape[1], _p(q_weight), _p(k_weight), _dt(wt) if wt is not None else 0, float(eps),
+        float(temp_coef), int(temp_every), _p(row_pos), _p(row_seq), _p(page_table) if store else None, max_pages, n_pages,
+        _p(k_cache) if store else None, _p(v_cache) if store else None, cache_dt, n, heads_q, heads_kv, head_dim,
+        1 if store else 0, 1 if values_from_keys else 0, _stream()))
+    return q
+
+
+def attention_shared_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor,
+                           row_pos: torch.Tensor, row_seq: torch.Tensor, heads_q: int, heads_kv: int, head_dim: int,
+                           v_dim: int, scale: float, r1: Optional[torch.Tensor], r2: Optional[torch.Tensor]) -> torch.Tensor:
+    """O[row, g, c] = sum_j P_g(row, j) V_c(j): every query head's causal softmax (scores times ``scale``
+    minus r1_g ln(1 + r2_g distance)) applied to the values of every key/value head; float32
+    [rows, heads_q, heads_kv, v_dim].  One wave per (row, g, c)."""
+    _dev(q, k_cache, v_cache, page_table, row_pos, row_seq, r1, r2)
+    n = q.shape[0]
+    if q.dim() != 2 or q.shape[1] != heads_q * head_dim:
+        raise KernelLibraryError(f"queries must be [rows, {heads_q * head_dim}]")
+    _check_cache_kv(k_cache, v_cache, heads_kv, head_dim, v_dim)
+    _check_rows(row_pos, row_seq, page_table, n)
+    if (r1 is None) != (r2 is None):
+        raise KernelLibraryError("the distance bias needs both of its numbers a head")
+    if r1 is not None:
+        _f32_vec(r1, heads_q, "r1")
+        _f32_vec(r2, heads_q, "r2")
+    out = torch.empty((n, heads_q, heads_kv, v_dim), dtype=torch.float32, device=q.device)
+    check(library.core().sb_attention_shared(_p(out), _p(q), _dt(q), _p(k_cache), _p(v_cache), _dt(k_cache), _p(page_table),
+                                             page_table.shape[1], k_cache.shape[0], _p(row_pos), _p(row_seq), n, heads_q,
+                                             heads_kv, head_dim, v_dim, float(scale), _p(r1), _p(r2), _stream()))
+    return out
+
+
+def head_mix(o: torch.Tensor, mix: Optional[torch.Tensor], out_dtype: torch.dtype) -> torch.Tensor:
+    """out[row, h] = sum_g mix[h, g] o[row, g, kv(h)] for ``o`` float32 [rows, heads_q, heads_kv, v_dim]
+    (``mix`` None: the identity); [rows, heads_q * v_dim] in ``out_dtype``."""
+    _dev(o, mix)
+    if o.dtype != torch.float32 or o.dim() != 4:
+        raise KernelLibraryError("the heads' results must be float32 [rows, heads_q, heads_kv, v_dim]")
+    n, hq, hkv, vd = o.shape
+    if mix is not None and tuple(mix.shape) != (hq, hq):
+        raise KernelLibraryError(f"the heads' mixing matrix must be [{hq}, {hq}]")
+    out = torch.empty((n, hq * vd), dtype=out_dtype, device=o.device)
+    check(library.core().sb_head_mix(_p(out), _dt(out), _p(o), _p(mix), _dt(mix) if mix is not None else 0, n, hq, hkv, vd,
+                                     _stream()))
+    return out
+
+
+def attention_shared(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor, ctx,
+                     heads_q: int, heads_kv: int, head_dim: int, v_dim: int, scale: float, r1: Optional[torch.Tensor],
+                     r2: Optional[torch.Tensor], mix: Optional[torch.Tensor], out_dtype: torch.dtype,
+                     fast: bool = True) -> torch.Tensor:
+    """Attention of a step's rows over the cache with a distance bias and the heads' weights mixed by
+    ``mix`` [heads_q, heads_q]: every query head's weights against every key/value head's values, then the
+    mix of the results; [rows, heads_q * v_dim] in ``out_dtype``."""
+    o = attention_shared_plain(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_seq, heads_q, heads_kv, head_dim,
+                               v_dim, scale, r1, r2)
+    return head_mix(o, mix, out_dtype)

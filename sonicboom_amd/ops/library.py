@@ -68,6 +68,18 @@ _CORE_SIGNATURES = {
     "sb_moe_router": [_P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _P],
     "sb_swish_clamp_mul": [_P, _I, _P, _I, _I, _F, _F, _P],
     "sb_moe_product": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _F, _P],
+    "sb_moe_route_scored": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
+    "sb_moe_router_scored": [_P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _P],
+    "sb_time_conv_max_taps": [],
+    "sb_time_conv": [_P, _I, _I, _P, _I, _I, _P, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+    "sb_time_conv_keep": [_P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _P],
+    "sb_state_scan_max_rows": [],
+    "sb_state_scan_max_cols": [],
+    "sb_ssd_scan": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "sb_delta_scan": [_P, _I, _I, _P, _I, _P, _I, _P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P],
+    "sb_qk_rownorm_store": [_P, _I, _P, _I, _P, _P, _I, _F, _F, _I, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+    "sb_attention_shared": [_P, _P, _I, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _P, _P, _P],
+    "sb_head_mix": [_P, _I, _P, _P, _I, _I, _I, _I, _I, _P],
     "sb_latent_attention_bf16": [_P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _P, _P, _I, _P],
 }
 # Entry points of later kernels; declared when the library has them.

@@ -2,4 +2,5 @@
 from .base import (CATEGORIES, Branch, KVSpec, Mixer, Part, RowsSpec, Runtime, StateSpec, build_part,  # noqa: F401
                    register_part, registered_parts)
 from .spec import ModelSpec, OrderEntry, PartSpec, TensorSpec  # noqa: F401
-from . import attention, block, embedding, ffn, latent_attention, moe, norm, position, recurrent  # noqa: F401
+from . import (attention, block, embedding, ffn, latent_attention, moe, norm, position, recurrent,  # noqa: F401
+               shared_attention, state_space)

@@ -14,7 +14,8 @@ copy in the activation type, ``ctx`` the step's
                 and, for encodings that are not rotary, ``apply(qkv, ctx, heads_q,
                 heads_kv, head_dim)`` acting in place on float32 qkv rows;
                 ``score_scale`` multiplies the attention scale.
-* **mixer**     ``cache_spec() -> KVSpec | RowsSpec | None``, ``state_spec() -> StateSpec | None``,
+* **mixer**     ``cache_spec() -> KVSpec | RowsSpec | None``, ``state_spec() -> StateSpec | {name: StateSpec} | None``
+                (one state: ``binding.state``; several by name: ``binding.states[name]``),
                 ``forward(h, x, ctx, binding)`` adds the mixer's output into ``x``.
 * **ffn**       ``forward(h, x, ctx)`` adds the feed-forward's output into ``x``.
                 Mixers and feed-forwards may set ``fuses_norm`` (their ``forward`` then
@@ -26,7 +27,9 @@ copy in the activation type, ``ctx`` the step's
                 blocks that norm a sublayer's output need it.
 * **block**     ``mixer`` attribute and ``forward(x, ctx, binding, h=None, next_norm=None)``;
                 optionally ``first_norm``, the norm the block starts with (the block before
-                may then hand over ``h`` = first_norm(x) from its last pass), and calls of
+                may then hand over ``h`` = first_norm(x) from its last pass), ``state_specs() ->
+                {name: StateSpec}`` for per-sequence state the block itself keeps (it finds it at
+                ``binding.states["block.<name>"]``), and calls of
                 ``ctx.trace(name, x)`` after its mixer and feed-forward when that is set.
 * **embedding** ``forward(ids, ctx) -> x`` (``ctx.row_pos`` for embeddings that add a position's row)
 * **head**      ``forward(h) -> float32 logits [rows, vocab]``
@@ -121,7 +124,7 @@ class Mixer(Part):
     def cache_spec(self) -> "Optional[KVSpec | RowsSpec]":
         return None
 
-    def state_spec(self) -> Optional[StateSpec]:
+    def state_spec(self) -> "Optional[StateSpec | Dict[str, StateSpec]]":
         return None
 
     def forward(self, h, x, ctx, binding) -> None:

@@ -5,7 +5,10 @@ optional post-norms): x += mixer(norm(x)); x += ffn(norm(x)).  Mixer and
 feed-forward add their result into the float32 residual stream themselves,
 which lets their last projection fuse the addition (and a multiplier of the
 branch, the ``out_scale`` of their specs).  A block may have no feed-forward:
-it is then the first sublayer alone.
+it is then the first sublayer alone.  With ``input_taps`` the mixer reads h + conv(h) in place of
+h = norm(x): a causal convolution over time on every channel of the normed stream (taps
+[width, input_taps], the last on the current token, zeros before the sequence's start), whose last
+input_taps - 1 inputs are per-sequence state of the block.
 
 ``outnorm``: the sublayers read the stream as it is and the norm sits on what they give back:
 x += norm(mixer(x)); x += norm(ffn(x)).  The mixer and the feed-forward hand their result over
@@ -14,18 +17,29 @@ stream in the activation type for the sublayer that reads it next.
 """
 from __future__ import annotations
 
+import torch
+
 from .. import ops
-from .base import Branch, Part, register_part
-from .spec import PartSpec
+from .base import Branch, Part, StateSpec, register_part
+from .spec import PartSpec, TensorSpec
 
 
-def prenorm_block_spec(mixer_norm: PartSpec, mixer: PartSpec, ffn_norm: PartSpec = None, ffn: PartSpec = None) -> PartSpec:
+def prenorm_block_spec(mixer_norm: PartSpec, mixer: PartSpec, ffn_norm: PartSpec = None, ffn: PartSpec = None,
+                       input_conv_name: str = None, input_taps: int = 0, width: int = 0) -> PartSpec:
+    """``input_conv_name``: the tensor [width, input_taps] of the convolution over time that the
+    mixer's input passes (h + conv(h))."""
     parts = {"mixer_norm": mixer_norm, "mixer": mixer}
     if ffn is not None:
         if ffn_norm is None:
             raise ValueError("a block with a feed-forward needs the norm before it")
         parts.update(ffn_norm=ffn_norm, ffn=ffn)
-    return PartSpec("block", "prenorm", {}, {}, parts)
+    params, tensors = {}, {}
+    if input_conv_name is not None:
+        if input_taps < 2 or width <= 0:
+            raise ValueError("a convolution on the mixer's input needs at least two taps and the stream's width")
+        params = {"input_taps": int(input_taps), "width": int(width)}
+        tensors = {"input_conv": TensorSpec(input_conv_name, (width, input_taps), init=(0.0, 0.1))}
+    return PartSpec("block", "prenorm", params, tensors, parts)
 
 
 @register_part("block", "prenorm")
@@ -39,6 +53,16 @@ class PreNormBlock(Part):
         self.mixer = parts["mixer"]
         self.ffn_norm = parts.get("ffn_norm")
         self.ffn = parts.get("ffn")              # None: the block is its mixer's sublayer alone
+        self.input_taps = int(spec.params.get("input_taps", 0) or 0)
+        self.input_conv = tensors.get("input_conv") if self.input_taps else None
+        if self.input_taps and self.input_taps > ops.time_conv_max_taps():
+            raise ValueError(f"{self.input_taps} taps are more than the convolution kernel's {ops.time_conv_max_taps()}")
+
+    def state_specs(self):
+        """The last taps - 1 inputs of the convolution on the mixer's input, a row of the stream's width each."""
+        if not self.input_taps:
+            return {}
+        return {"input_conv": StateSpec((self.input_taps - 1, int(self.spec.params["width"])), torch.float32)}
 
     def forward(self, x, ctx, binding, h=None, next_norm=None):
         """Run the block on the residual stream ``x`` in place.  ``h`` is mixer_norm(x) when the
@@ -49,6 +73,8 @@ class PreNormBlock(Part):
         act = self.rt.act_dtype
         if h is None:
             h = self.mixer_norm.forward(x, act)
+        if self.input_conv is not None:
+            h = ops.time_conv(h, self.input_conv, None, binding.states["block.input_conv"], ctx, act, residual=True)
         f = None
         after = self.ffn_norm if self.ffn is not None else next_norm     # the norm that follows the mixer
         if getattr(self.mixer, "fuses_norm", False):

@@ -6,6 +6,11 @@
 
     expert(f) = W_down (g' sigmoid(alpha g') (u' + 1)),  g' = min(W_gate f, limit),
     u' = W_up f cut to [-limit, limit]                                  ("swish_clamp")
+    expert(f) = W_down (silu(W_gate f) W_up f)                          ("silu")
+
+With ``router_score`` "sigmoid" the scores are s = sigmoid(z), the ``top`` largest s are chosen and
+their weights are s times ``router_scale``, not renormalized.  ``shared_gate`` false: the expert
+that every row takes is added as it is (no sigmoid gate, no tensor for it).
 
 The router runs in float32 whatever the model's type (its matrix, with the shared expert's gate
 row under it, is kept in float32; one kernel makes the scores and the choice).  Choice and weights
@@ -28,15 +33,17 @@ from .base import Branch, Part, register_part
 from .linear import Linear
 from .spec import PartSpec, TensorSpec
 
-EXPERT_ACTIVATIONS = ("swish_clamp",)
+EXPERT_ACTIVATIONS = ("swish_clamp", "silu")
+ROUTER_SCORES = ("softmax_chosen", "sigmoid")
 
 
 def moe_ffn_spec(prefix: str, width: int, experts: int, top: int, inner: int, limit: float, alpha: float = 1.702,
                  shared_inner: int = 0, shared_limit: float = 0.0, activation: str = "swish_clamp",
                  names=("gate", "up", "down"), expert_prefix: str = "e{}.", router_name: str = "router",
-                 shared_prefix: str = "shared.", shared_gate_name: str = "shared.sg") -> PartSpec:
+                 shared_prefix: str = "shared.", shared_gate_name: str = "shared.sg", router_score: str = "softmax_chosen",
+                 router_scale: float = 1.0, shared_gate: bool = True) -> PartSpec:
     """``shared_inner`` > 0: an expert of that inner width that every row takes, times the sigmoid of
-    one more router row (``shared_gate_name``)."""
+    one more router row (``shared_gate_name``) unless ``shared_gate`` is false."""
     tensors = {"router": TensorSpec(prefix + router_name, (experts, width))}
     for e in range(experts):
         ep = prefix + expert_prefix.format(e)
@@ -48,10 +55,13 @@ def moe_ffn_spec(prefix: str, width: int, experts: int, top: int, inner: int, li
         tensors["shared.gate"] = TensorSpec(sp + names[0], (shared_inner, width))
         tensors["shared.up"] = TensorSpec(sp + names[1], (shared_inner, width))
         tensors["shared.down"] = TensorSpec(sp + names[2], (width, shared_inner))
-        tensors["shared.sg"] = TensorSpec(prefix + shared_gate_name, (1, width))
+        if shared_gate:
+            tensors["shared.sg"] = TensorSpec(prefix + shared_gate_name, (1, width))
     return PartSpec("ffn", "moe", {"width": width, "experts": experts, "top": top, "inner": inner, "limit": float(limit),
                                    "alpha": float(alpha), "shared_inner": int(shared_inner),
-                                   "shared_limit": float(shared_limit), "activation": activation}, tensors)
+                                   "shared_limit": float(shared_limit), "activation": activation,
+                                   "router_score": router_score, "router_scale": float(router_scale),
+                                   "shared_gate": bool(shared_gate)}, tensors)
 
 
 def _stack(mats):
@@ -71,14 +81,19 @@ class MoEFFN(Part):
         self.width, self.experts, self.top, self.inner = int(p["width"]), int(p["experts"]), int(p["top"]), int(p["inner"])
         self.limit, self.alpha = float(p["limit"]), float(p.get("alpha", 1.702))
         self.shared_inner, self.shared_limit = int(p.get("shared_inner", 0)), float(p.get("shared_limit", 0.0))
-        if p.get("activation", "swish_clamp") not in EXPERT_ACTIVATIONS:
+        self.activation = p.get("activation", "swish_clamp")
+        if self.activation not in EXPERT_ACTIVATIONS:
             raise ValueError(f"unknown expert activation {p.get('activation')!r}; known: {EXPERT_ACTIVATIONS}")
+        self.router_score, self.router_scale = p.get("router_score", "softmax_chosen"), float(p.get("router_scale", 1.0))
+        if self.router_score not in ROUTER_SCORES:
+            raise ValueError(f"unknown kind of router score {self.router_score!r}; known: {ROUTER_SCORES}")
+        self.shared_gate = bool(p.get("shared_gate", True)) and bool(int(p.get("shared_inner", 0)))
         if not 0 < self.top <= self.experts:
             raise ValueError(f"{self.top} choices of {self.experts} experts")
         if self.top > ops.MOE_MAX_TOP:
             raise ValueError(f"{self.top} choices a row are more than the router kernel's {ops.MOE_MAX_TOP}")
         rows = [tensors["router"].float()]
-        if self.shared_inner:
+        if self.shared_gate:
             rows.append(tensors["shared.sg"].float().reshape(1, self.width))
         self.router = torch.cat(rows, dim=0).contiguous()        # float32, the shared expert's gate row last
         self.w_in = ops.MoEWeight(_stack([torch.cat([tensors[f"e{e}.gate"], tensors[f"e{e}.up"]], dim=0)
@@ -91,7 +106,8 @@ class MoEFFN(Part):
             g, u = tensors["shared.gate"], tensors["shared.up"]
             if g.dtype != u.dtype:
                 g, u = g.float(), u.float()
-            self.s_in = Linear(torch.cat([g, u], dim=0), None, rt.fast_kernels)
+            # (the plain silu pair is the gated product of the dense feed-forwards, applied in the product's epilogue)
+            self.s_in = Linear(torch.cat([g, u], dim=0), None, rt.fast_kernels, gated=self.activation == "silu")
             self.s_out = Linear(tensors["shared.down"], None, rt.fast_kernels)
 
     def produce(self, h, ctx):
@@ -99,15 +115,19 @@ class MoEFFN(Part):
         gate, for the pass that adds them up."""
         act = self.rt.act_dtype
         n = h.shape[0]
-        ids, weights = ops.moe_router(h, self.router, self.experts, self.top, has_gate=bool(self.shared_inner))
+        ids, weights = ops.moe_router(h, self.router, self.experts, self.top, has_gate=self.shared_gate,
+                                      score=self.router_score, score_scale=self.router_scale)
         plan = ops.moe_plan(ids, self.experts)
-        mid = ops.moe_product(h, self.w_in, plan, self.top, act, self.limit, self.alpha)       # [n * top, inner]
+        mid = ops.moe_product(h, self.w_in, plan, self.top, act, self.limit, self.alpha, pair=self.activation)   # [n * top, inner]
         out = ops.moe_product(mid, self.w_out, plan, 1, torch.float32)                         # [n * top, width]
         branch = Branch(out.view(n, self.top, self.width), by_row=True, part_weights=weights[:, : self.top])
         if self.shared_inner:
-            smid = ops.swish_clamp_mul(self.s_in(h, torch.float32), act, self.shared_limit, self.alpha)
+            if self.activation == "silu":
+                smid = self.s_in.gated_product(h, act)
+            else:
+                smid = ops.swish_clamp_mul(self.s_in(h, torch.float32), act, self.shared_limit, self.alpha)
             branch.extra = self.s_out(smid, torch.float32)
-            branch.extra_weights = weights[:, self.top:]
+            branch.extra_weights = weights[:, self.top:] if self.shared_gate else None
         return branch
 
     def forward(self, h, x, ctx, then_norm=None):

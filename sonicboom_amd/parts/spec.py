@@ -22,7 +22,8 @@ class TensorSpec:
     ``kind`` is "float" (kept in bfloat16, or in float32 when stored so or when
     the whole model runs in 32-bit) or "int" (kept as int32).  ``init`` is
     (mean, std) of the seeded random mode.  An ``optional`` tensor may be
-    absent from the file; the part then receives None.
+    absent from the file; the part then receives None.  An axis of ``shape`` given as -1 takes
+    whatever size the file has (seeded random weights need every axis).
     """
     name: str
     shape: Tuple[int, ...]

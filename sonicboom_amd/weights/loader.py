@@ -75,7 +75,8 @@ def check_against_spec(found: Dict[str, tuple], wanted: List[TensorSpec], ignora
                 problems.append(f"missing tensor: {t.name} (the model wants shape {list(t.shape)})")
             continue
         dtype, shape = found[t.name]
-        if tuple(shape) != tuple(t.shape):
+        # an axis the spec gives as -1 takes the size the file has (a rank that only the tensors tell)
+        if len(shape) != len(t.shape) or any(w != -1 and w != n for w, n in zip(t.shape, shape)):
             problems.append(f"tensor shape mismatch: {t.name} (the file has {list(shape)} {dtype}, "
                             f"the model wants {list(t.shape)})")
         elif (t.kind == "float" and dtype not in _FLOAT) or (t.kind == "int" and dtype not in _INT):

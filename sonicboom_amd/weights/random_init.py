@@ -40,6 +40,12 @@ def _draw(seed: int, index: int, shape, mean: float, std: float, device=None) ->
     return random_stream.draw(seed, index, shape, mean, std)
 
 
+def _whole_shape(t) -> None:
+    if any(n < 0 for n in t.shape):
+        raise ValueError(f"tensor {t.name}: the configuration leaves an axis to the file ({list(t.shape)}); "
+                         "random weights need every size")
+
+
 def random_arrays(spec: ModelSpec, seed: int, device=None) -> Dict[str, np.ndarray]:
     """float32 arrays (int32 zeros for integer tables) for every tensor of the spec."""
     return dict(iter_random_arrays(spec, seed, device))
@@ -49,6 +55,7 @@ def iter_random_arrays(spec: ModelSpec, seed: int, device=None):
     """(name, array) for every tensor of the spec, one at a time: float32 arrays, int32 zeros for
     integer tables.  ``device``: a GPU that draws the large tensors (same bits as the host)."""
     for i, t in enumerate(spec.all_tensors()):
+        _whole_shape(t)
         if t.kind == "int":
             yield t.name, np.zeros(t.shape, dtype=np.int32)
         else:
@@ -106,6 +113,7 @@ def random_source(spec: ModelSpec, seed: int, dtype: str, device, stored=None):
 
     def make(name):
         i, t = specs[name]
+        _whole_shape(t)
         if t.kind == "int":
             return torch.zeros(t.shape, dtype=torch.int32, device=device)
         mean, std = t.init
