@@ -36,7 +36,8 @@ one prompt step and one decode step with what it reaches of its roofline (bytes 
 8 TB/s, or flops over the dense bf16 peak, whichever is the larger time).  A table goes to standard
 error, one JSON line to standard output.  ``--design tatelorn`` puts the Tatelorn design (blocks that
 norm what their sublayers give back, attention with head norms, capped scores and a sink, routed
-experts) in the Rasizen design's place: eight layers, the first with a dense gated feed-forward, the
+experts) in the Rasizen design's place (``--design nalasun``: the Nalasun design, state-space and delta-rule
+recurrences, attention with shared head weights and routed experts behind short convolutions): eight layers, the first with a dense gated feed-forward, the
 others with eight experts of which a row takes two plus a shared one, so that a row passes as many
 feed-forward weights as in the Qwen2.5 design beside it, and the same heads.
 
@@ -262,7 +263,7 @@ def main() -> int:
     ap.add_argument("--prompt", type=int, default=PROMPT, help="cached prompt tokens per sequence")
     ap.add_argument("--context", type=int, default=CONTEXT, help="cache size per sequence")
     ap.add_argument("--workload", choices=("steady", "mixed", "forms", "designs"), default="steady")
-    ap.add_argument("--design", choices=("rasizen", "tatelorn"), default="rasizen",
+    ap.add_argument("--design", choices=("rasizen", "tatelorn", "nalasun"), default="rasizen",
                     help="--workload designs: the design that runs beside the Qwen2.5 design")
     ap.add_argument("--design-sizes", default="2048,4096",
                     help="--workload designs: the widths of the layer sizes to run, comma separated")
@@ -690,6 +691,29 @@ def tatelorn_sizes(width, n_layers=8, vocab=32768, experts=8, top=2):
             "embedding": {"scale": width ** 0.5}, "norm": {"eps": 1e-6}, "layers": layers}
 
 
+def nalasun_sizes(width, vocab=32768, experts=8, top=2):
+    """Layer sizes in the manner of a real model of this width, eight layers: state-space layers of 2 widths in
+    heads of 64 channels with a state of 128 rows and eight groups, attention with heads of 128 (a quarter of them
+    key/value heads), delta-rule layers with heads of 128 x 128, every layer's mixer behind a convolution of four taps;
+    `experts` experts of one width of which a row takes `top`, and a shared expert that brings a row's feed-forward
+    weights to those of the dense layer of the Qwen2.5 design beside it."""
+    heads = width // 128
+    inner = (8 * width // 3 + 255) // 256 * 256
+    routed = {"kind": "moe", "router": {"experts": experts, "top": top, "scale": 1.5}, "expert": {"ff": width},
+              "shared": {"ff": max(256, inner - top * width)}}
+    ssm = {"type": "mamba2", "mixer": {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 8}}
+    att = {"type": "attention", "mixer": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128,
+                                          "scale": 128 ** -0.5, "q_temp": {"coef": 0.5, "every": 256}}}
+    delta = {"type": "channel_delta", "mixer": {"heads": heads, "kv_heads": max(1, heads // 2), "dim": 128, "vdim": 128, "conv": 4,
+                                                "decay_rank": 64, "gate_rank": 64}}
+    layers = [dict(layer, mlp=routed) for layer in (ssm, att, att, delta, ssm, att, delta, ssm)]
+    return {"architecture": "Nalasun", "vocab": vocab, "width": width, "max_positions": 1 << 16, "norm": {"eps": 1e-6},
+            "canon": {"taps": 3}, "layers": layers}
+
+
+VECTOR_F32_FLOPS = 157.3e12      # the vector units' float32 peak, against which the recurrences' scans are priced
+
+
 class AllOpsTimer:
     """Times every launching function of ``sonicboom_amd.ops`` between two events, summed by
     (function, what tells its calls apart: a product's matrix, the rows)."""
@@ -697,10 +721,12 @@ class AllOpsTimer:
     SKIP = ("pack_weight", "read_bandwidth", "random_normal", "attention_row_tile", "attention_row_tiles",
             "attention_tall_ok", "attention_mfma_ok", "attention_decode_rope_ok", "gate_code", "reduce_resid_norm_ok",
             "attention_decode_pages_per_wave", "gemm_tile_shape", "gemm_few_rows_kernel", "mingru_chunk_rows",
-            "loaded_paths", "check", "latent_attention_mfma_ok", "capped_attention_mfma_ok", "moe_max_top", "moe_plan")
+            "loaded_paths", "check", "latent_attention_mfma_ok", "capped_attention_mfma_ok", "moe_max_top", "moe_plan",
+            "time_conv_max_taps", "state_scan_limits", "shared_attention_mfma_ok")
     INNER = ("attention_plain", "attention_decode_mfma", "attention_prefill_mfma", "latent_attention_plain",
              "latent_attention_mfma", "attention_capped_plain", "attention_capped_mfma",
-             "moe_product_plain")      # called by the dispatchers that are timed themselves
+             "moe_product_plain", "attention_shared_plain", "attention_shared_mfma",
+             "head_mix")               # called by the dispatchers that are timed themselves
 
     def __init__(self):
         self.records, self._saved = [], {}
@@ -729,6 +755,8 @@ class AllOpsTimer:
                         label = f"{_name} {n}x{k}"
                     elif _name == "head_product":
                         label = f"{_name} {tuple(args[1].shape)}"
+                    elif _name == "time_conv":
+                        label = f"{_name} {args[1].shape[0]}"
                     elif _name == "moe_product":
                         label = f"{_name} {args[1].experts}x{args[1].n_out}x{args[1].n_in}{' gated' if args[1].gated else ''}"
                     self.records.append((label, e0, e1))
@@ -805,6 +833,23 @@ def design_roofline(label, us, calls, rows, depth, batch, width, cfgs):
         pairs = rows * (cfgs["top"] if e > 1 else 1)
         nbytes = 2 * min(e, pairs) * m * n * k + 2 * pairs * (k + n)
         flops = 2 * pairs * m * n * k
+    elif label.startswith("time_conv"):
+        nbytes = rows * int(label.split()[1]) * (4 + 4)
+    elif label == "ssd_scan":
+        h, n, p = cfgs["ssd"]
+        nbytes = rows * (4 * 3 * h * p + 4 * h) + (2 * batch * 4 * h * n * p if decode else 0)
+        flops, peak_f = rows * h * n * p * 4, VECTOR_F32_FLOPS
+    elif label == "delta_scan":
+        h, d, e = cfgs["delta"]
+        nbytes = rows * (4 * (2 * h * d + 3 * h * e) + 2 * h * e) + (2 * batch * 4 * h * d * e if decode else 0)
+        flops, peak_f = rows * h * d * e * 7, VECTOR_F32_FLOPS
+    elif label == "qk_rownorm_store":
+        nbytes = rows * (H * 128 + cfgs["kvw"]) * (4 + 2) + rows * cfgs["kvw"] * 2
+    elif label == "attention_shared":
+        pairs = batch * depth if decode else rows * (rows + 1) // 2
+        g = cfgs["kvw"] // 128
+        flops = 2 * pairs * H * 128 * (1 + g)
+        nbytes = (batch * depth if decode else rows) * 2 * 2 * cfgs["kvw"] + 2 * rows * H * 128 * 2
     if nbytes is None and flops is None:
         return None, ""
     tb, tf = (nbytes or 0) / peak_b, (flops or 0) / peak_f
@@ -820,13 +865,15 @@ def design_comparison(a) -> int:
     rng = np.random.default_rng(0)
     out, table = {}, []
     for width in (int(v) for v in a.design_sizes.split(",")):
-        beside = ("rasizen", rasizen_sizes(width)) if a.design == "rasizen" else ("tatelorn", tatelorn_sizes(width))
+        beside = {"rasizen": rasizen_sizes, "tatelorn": tatelorn_sizes, "nalasun": nalasun_sizes}[a.design]
+        beside = (a.design, beside(width))
         for design, cfg in (beside, ("qwen2", qwen_sizes(width))):
             model = DecoderModel.from_random(cfg, seed=0, dtype="bfloat16", device="cuda:0")
             heads = width // 128
             cfgs = {"heads": heads, "rank": 512, "rot": 64, "window": 4096 if design == "rasizen" else 1 << 30,
                     "gru": 2 * width, "ff": 4 * width, "kvw": max(1, heads // 4) * 128,
-                    "vocab": cfg.get("vocab", cfg.get("vocab_size")), "top": 2}
+                    "vocab": cfg.get("vocab", cfg.get("vocab_size")), "top": 2,
+                    "ssd": (2 * width // 64, 128, 64), "delta": (heads, 128, 128)}
             eng = Engine(model, (a.prompt + a.steps + a.warmup + 128) * (a.batch + 1), max_positions=0)
             prompt = [int(t) for t in rng.integers(0, cfg.get("vocab", cfg.get("vocab_size")), size=a.prompt)]
 
