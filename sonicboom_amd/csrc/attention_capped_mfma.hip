@@ -14,6 +14,11 @@
 //         row r of an S^T tile stands for key 8 (r / 4) + 4 t + r % 4 of a half page (t the tile), so
 //         the eight probabilities a lane holds after two tiles are eight consecutive keys.
 //
+// Two further forms of the score and of the result, for mixers whose heads share their weights:
+// a bias by the logarithm of the distance, score - r1[h] ln(1 + r2[h] (p - j)) (`dist_r1`, `dist_r2`), and
+// `all_values`: every query head's weights applied to the values of every kv head, not its own alone
+// (the grid then holds a block per value head too, and the result is [rows, heads_q, heads_kv, dv]).
+//
 // Softmax in float32, running maximum and sum per query column, scores kept times log2(e) so that the
 // weights are powers of two; a sink starts the maximum at 0 and the sum at 1.  Steps of few rows
 // share the pages of a sequence out over `chunks` blocks, which leave (unnormed result, maximum,
@@ -60,6 +65,8 @@ struct Args {
   const int32_t *row_pos, *tiles;
   int n_rows, heads_q, heads_kv;
   float scale, softcap; int window, sink, chunk_pages;
+  const float *dist_r1, *dist_r2;      // [heads_q] or NULL: the bias by the distance's logarithm
+  int all_values;                      // 1: blockIdx.y also counts the kv head whose values are read
   unsigned round_blocks;       // blocks the GPU takes one of per CU
 };
 
@@ -78,7 +85,12 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
   __shared__ int page_lds[kPagesInLds];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, g = lane >> 4;
   const int group = a.heads_q / a.heads_kv, zgroups = (group + NW - 1) / NW;
-  const int kvh = blockIdx.y / zgroups, hz = blockIdx.y % zgroups;
+  const int kv_blocks = a.heads_kv * zgroups;
+  const int vh_own = a.all_values ? int(blockIdx.y) / kv_blocks : -1;       // the kv head whose values this block reads
+  const int by = int(blockIdx.y) % kv_blocks;
+  const int kvh = by / zgroups, hz = by % zgroups;
+  const int vh = a.all_values ? vh_own : kvh;
+  const int out_heads = a.all_values ? a.heads_q * a.heads_kv : a.heads_q;   // heads of the result's rows
   const int hg = hz * NW + wave;                  // the wave's head within the group
   const bool has_head = hg < group;
   const int h = kvh * group + (has_head ? hg : 0);
@@ -120,6 +132,8 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
   const float cap_arg = a.softcap > 0.0f ? a.scale * 2.0f * kLog2e / a.softcap : 0.0f;      // the scale rides along
   // scores are kept times log2(e), so that the weights are powers of two: the sink's score stays 0
   const float scale2 = a.scale * kLog2e, cap2 = a.softcap * kLog2e;
+  // r1 ln(1 + r2 d) log2(e) = r1 log2(1 + r2 d): the hardware's logarithm is the one to base two
+  const float r1 = (a.dist_r1 && has_head) ? a.dist_r1[h] : 0.0f, r2 = (a.dist_r2 && has_head) ? a.dist_r2[h] : 0.0f;
 
   // two pages' loads are in flight while a third is attended (a CU holds few of these blocks: a page's
   // round trip to memory would otherwise show once per page)
@@ -146,7 +160,7 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
       if (page >= a.n_pages) page = -1;
     }
     const uint4 *kp = reinterpret_cast<const uint4 *>(a.k_cache + (size_t(max(page, 0)) * a.heads_kv + kvh) * SB_PAGE * DK);
-    const uint4 *vp = reinterpret_cast<const uint4 *>(a.v_cache + (size_t(max(page, 0)) * a.heads_kv + kvh) * SB_PAGE * DV);
+    const uint4 *vp = reinterpret_cast<const uint4 *>(a.v_cache + (size_t(max(page, 0)) * a.heads_kv + vh) * SB_PAGE * DV);
 #pragma unroll
     for (int i = 0; i < kKeyLoads; ++i) {
       const int idx = tid + i * kThreads;
@@ -218,6 +232,13 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
           else v = s[t][i] * scale2;
           sc[4 * t + i] = v;
         }
+      if (a.dist_r1) {        // uniform over the block
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float dist = float(max(q_pos - (first + 8 * g + e), 0));
+          sc[e] -= r1 * __builtin_amdgcn_logf(fmaf(r2, dist, 1.0f));
+        }
+      }
       if (!whole) {           // uniform over the block: only pages on the diagonal or at a window's edge test their scores
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -273,7 +294,7 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
   const int row = r0 + col;
   if (a.out) {
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-    bf16_t *dst = a.out + (size_t(row) * a.heads_q + h) * DV;
+    bf16_t *dst = a.out + (size_t(row) * out_heads + (a.all_values ? h * a.heads_kv + vh : h)) * DV;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       uint2 w;
@@ -282,7 +303,7 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
       *reinterpret_cast<uint2 *>(dst + 16 * dt + 4 * g) = w;
     }
   } else {
-    const size_t at = (size_t(chunk) * a.n_rows + row) * a.heads_q + h;
+    const size_t at = (size_t(chunk) * a.n_rows + row) * out_heads + (a.all_values ? h * a.heads_kv + vh : h);
     float *dst = a.part_o + at * DV;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
@@ -344,11 +365,33 @@ extern "C" int sb_cattn_tile_rows(void) { return kTile; }
 // are shared out over that many blocks of chunk_pages pages each (chunks * chunk_pages >= max_pages)
 // and merged; part_o f32 [chunks * rows * heads_q * dv] and part_ml f32 [chunks * rows * heads_q * 2]
 // are the scratch for that.
+extern "C" int sb_cattn_shared_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
+                                    const int32_t *page_table, int max_pages, int n_pages, const int32_t *row_pos,
+                                    const int32_t *tiles, int n_tiles, int n_rows, int heads_q, int heads_kv, float scale,
+                                    int window, float softcap, int sink, int chunks, int chunk_pages, float *part_o,
+                                    float *part_ml, const float *dist_r1, const float *dist_r2, int all_values,
+                                    void *stream);
+
 extern "C" int sb_cattn_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
                              const int32_t *page_table, int max_pages, int n_pages, const int32_t *row_pos,
                              const int32_t *tiles, int n_tiles, int n_rows, int heads_q, int heads_kv, float scale,
                              int window, float softcap, int sink, int chunks, int chunk_pages, float *part_o,
                              float *part_ml, void *stream) {
+  return sb_cattn_shared_bf16(out, q, k_cache, v_cache, page_table, max_pages, n_pages, row_pos, tiles, n_tiles, n_rows,
+                              heads_q, heads_kv, scale, window, softcap, sink, chunks, chunk_pages, part_o, part_ml, nullptr,
+                              nullptr, 0, stream);
+}
+
+// The same with the bias r1[h] ln(1 + r2[h] distance) taken off every score (dist_r1, dist_r2 f32 [heads_q], or both
+// NULL) and, with all_values, every query head's weights applied to the values of every kv head: out bf16
+// [rows, heads_q, heads_kv, dv], the scratch heads_kv times as large.
+extern "C" int sb_cattn_shared_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
+                                    const int32_t *page_table, int max_pages, int n_pages, const int32_t *row_pos,
+                                    const int32_t *tiles, int n_tiles, int n_rows, int heads_q, int heads_kv, float scale,
+                                    int window, float softcap, int sink, int chunks, int chunk_pages, float *part_o,
+                                    float *part_ml, const float *dist_r1, const float *dist_r2, int all_values,
+                                    void *stream) {
+  SB_REQUIRE((dist_r1 == nullptr) == (dist_r2 == nullptr), "sb_cattn_bf16: the distance bias needs both of its numbers");
   SB_REQUIRE(out && q && k_cache && v_cache && page_table && row_pos && tiles, "sb_cattn_bf16: null pointer");
   SB_REQUIRE(n_tiles >= 0 && n_rows >= 0 && heads_q > 0 && heads_kv > 0 && max_pages > 0 && n_pages > 0 && window >= 0,
              "sb_cattn_bf16: bad sizes tiles=%d rows=%d heads=%d/%d", n_tiles, n_rows, heads_q, heads_kv);
@@ -359,7 +402,9 @@ extern "C" int sb_cattn_bf16(void *out, const void *q, const void *k_cache, cons
              "sb_cattn_bf16: %d chunks of %d pages do not cover %d pages, or have no scratch", chunks, chunk_pages, max_pages);
   if (n_tiles == 0 || n_rows == 0) return SB_OK;
   const int group = heads_q / heads_kv, zgroups = (group + NW - 1) / NW;
-  SB_SUPPORT((long long)heads_kv * zgroups <= 65535 && chunks <= 65535, "sb_cattn_bf16: too many heads or chunks for one grid");
+  const int value_heads = all_values ? heads_kv : 1;
+  SB_SUPPORT((long long)heads_kv * zgroups * value_heads <= 65535 && chunks <= 65535,
+             "sb_cattn_bf16: too many heads or chunks for one grid");
   hipStream_t s = (hipStream_t)stream;
   Args a;
   a.out = chunks == 1 ? (bf16_t *)out : nullptr;
@@ -369,10 +414,12 @@ extern "C" int sb_cattn_bf16(void *out, const void *q, const void *k_cache, cons
   a.n_rows = n_rows; a.heads_q = heads_q; a.heads_kv = heads_kv; a.scale = scale; a.softcap = softcap;
   a.window = window; a.sink = sink; a.chunk_pages = chunks == 1 ? 0 : chunk_pages;
   a.round_blocks = unsigned(sb::cu_count());
-  capped_attention_kernel<<<dim3(n_tiles, heads_kv * zgroups, chunks), kThreads, 0, s>>>(a);
+  a.dist_r1 = dist_r1; a.dist_r2 = dist_r2; a.all_values = all_values ? 1 : 0;
+  capped_attention_kernel<<<dim3(n_tiles, heads_kv * zgroups * value_heads, chunks), kThreads, 0, s>>>(a);
   int st = sb::check_launch("sb_cattn_bf16");
   if (st != SB_OK || chunks == 1) return st;
-  const size_t n = size_t(n_rows) * heads_q * DV;
-  merge_kernel<<<unsigned((n + 255) / 256), 256, 0, s>>>((bf16_t *)out, part_o, part_ml, chunks, size_t(n_rows) * heads_q);
+  const size_t n = size_t(n_rows) * heads_q * value_heads * DV;
+  merge_kernel<<<unsigned((n + 255) / 256), 256, 0, s>>>((bf16_t *)out, part_o, part_ml, chunks,
+                                                         size_t(n_rows) * heads_q * value_heads);
   return sb::check_launch("sb_cattn_merge");
 }

@@ -137,7 +137,7 @@ attention_shared_kernel(float *__restrict__ out, const TA *__restrict__ q, const
 
 // out[row, h, e] = sum over g of mix[h, g] * o[row, g, kv(h), e], in ascending g
 __global__ void __launch_bounds__(256)
-head_mix_kernel(void *__restrict__ out, int out_dtype, const float *__restrict__ o, const void *__restrict__ mix,
+head_mix_kernel(void *__restrict__ out, int out_dtype, const void *__restrict__ o, int o_dtype, const void *__restrict__ mix,
                 int mix_dtype, int heads_q, int heads_kv, int v_dim, size_t n) {
   const size_t idx = size_t(blockIdx.x) * 256 + threadIdx.x;
   if (idx >= n) return;
@@ -147,7 +147,7 @@ head_mix_kernel(void *__restrict__ out, int out_dtype, const float *__restrict__
   float acc = 0.0f;
   for (int g = 0; g < heads_q; ++g)
     acc = fmaf(mix ? ld_dyn(mix, mix_dtype, size_t(h) * heads_q + g) : (g == h ? 1.0f : 0.0f),
-               o[((row * heads_q + g) * heads_kv + vh) * v_dim + e], acc);
+               ld_dyn(o, o_dtype, ((row * heads_q + g) * heads_kv + vh) * v_dim + e), acc);
   st_dyn(out, out_dtype, idx, acc);
 }
 
@@ -203,15 +203,15 @@ extern "C" int sb_attention_shared(float *out, const void *q, int act_dtype, con
   return sb::check_launch("sb_attention_shared");
 }
 
-extern "C" int sb_head_mix(void *out, int out_dtype, const float *o, const void *mix, int mix_dtype, int n_rows, int heads_q,
-                           int heads_kv, int v_dim, void *stream) {
+extern "C" int sb_head_mix(void *out, int out_dtype, const void *o, int o_dtype, const void *mix, int mix_dtype, int n_rows,
+                           int heads_q, int heads_kv, int v_dim, void *stream) {
   SB_REQUIRE(out && o, "sb_head_mix: null pointer");
   SB_REQUIRE(n_rows >= 0 && heads_q > 0 && heads_kv > 0 && heads_q % heads_kv == 0 && v_dim > 0 && sb::valid_dtype(out_dtype) &&
-                 (!mix || sb::valid_dtype(mix_dtype)),
+                 sb::valid_dtype(o_dtype) && (!mix || sb::valid_dtype(mix_dtype)),
              "sb_head_mix: bad sizes rows=%d heads=%d kv=%d vdim=%d", n_rows, heads_q, heads_kv, v_dim);
   const size_t n = size_t(n_rows) * heads_q * v_dim;
   if (n == 0) return SB_OK;
-  head_mix_kernel<<<unsigned((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(out, out_dtype, o, mix, mix_dtype, heads_q, heads_kv,
-                                                                             v_dim, n);
+  head_mix_kernel<<<unsigned((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(out, out_dtype, o, o_dtype, mix, mix_dtype, heads_q,
+                                                                             heads_kv, v_dim, n);
   return sb::check_launch("sb_head_mix");
 }

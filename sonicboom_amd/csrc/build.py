@@ -50,7 +50,8 @@ ATTN_SOURCES = ["attention_mfma.hip"]
 CAPPED_ATTN_SOURCES = ["attention_capped_mfma.hip"]
 # (key size, value size) pairs of the capped attention kernels compiled ahead of time by build_all()
 PREBUILT_CAPPED_DIMS = ((64, 64), (128, 128), (128, 64), (192, 128), (256, 256), (64, 128), (32, 16), (48, 32), (16, 48), (32, 48),
-                        (16, 64), (32, 64), (64, 48), (16, 16), (16, 32), (32, 32))
+                        (16, 64), (32, 64), (64, 48), (16, 16), (16, 32), (32, 32)) + tuple(
+                            (n, n) for n in range(48, 257, 16) if n not in (64, 128, 256))      # values of the keys' size
 
 # Head sizes compiled ahead of time by build_all(): every size the kernels take.
 PREBUILT_HEAD_DIMS = tuple(range(16, 257, 16))

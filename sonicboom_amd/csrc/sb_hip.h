@@ -350,7 +350,7 @@ int sb_delta_scan(void *out, int out_dtype, int out_stride, const float *qkv, in
  *   key cache at the row's position and, with values_from_keys, k as it came into the value cache.
  * sb_attention_shared: O[row][g][c][:] = sum_j P_g(row, j) V_c(j), P_g the causal softmax of
  *   scale q_g . k_kv(g)(j) - r1[g] ln(1 + r2[g] (p - j)) (r1, r2 NULL: no bias); out f32.
- * sb_head_mix: out[row][h][:] = sum_g mix[h][g] O[row][g][kv(h)][:] (mix NULL: the identity). */
+ * sb_head_mix: out[row][h][:] = sum_g mix[h][g] O[row][g][kv(h)][:] (mix NULL: the identity); O of o_dtype. */
 int sb_qk_rownorm_store(void *q_out, int q_dtype, const float *qk, int row_stride, const void *q_w, const void *k_w,
                         int w_dtype, float eps, float temp_coef, int temp_every, const int32_t *row_pos,
                         const int32_t *row_seq, const int32_t *page_table, int max_pages, int n_pages, void *k_cache,
@@ -360,8 +360,8 @@ int sb_attention_shared(float *out, const void *q, int act_dtype, const void *k_
                         int cache_dtype, const int32_t *page_table, int max_pages, int n_pages_total,
                         const int32_t *row_pos, const int32_t *row_seq, int n_rows, int heads_q, int heads_kv,
                         int head_dim, int v_dim, float scale, const float *r1, const float *r2, void *stream);
-int sb_head_mix(void *out, int out_dtype, const float *o, const void *mix, int mix_dtype, int n_rows, int heads_q,
-                int heads_kv, int v_dim, void *stream);
+int sb_head_mix(void *out, int out_dtype, const void *o, int o_dtype, const void *mix, int mix_dtype, int n_rows,
+                int heads_q, int heads_kv, int v_dim, void *stream);
 
 /* ids[r] = index of the first maximum of logits[r,:].  Two stages over
  * sb_argmax_parts(vocab) parts of a row; part_val / part_idx hold n_rows * parts

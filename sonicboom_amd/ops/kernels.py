@@ -1616,17 +1616,65 @@ def attention_shared_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
 
 
 def head_mix(o: torch.Tensor, mix: Optional[torch.Tensor], out_dtype: torch.dtype) -> torch.Tensor:
-    """out[row, h] = sum_g mix[h, g] o[row, g, kv(h)] for ``o`` float32 [rows, heads_q, heads_kv, v_dim]
-    (``mix`` None: the identity); [rows, heads_q * v_dim] in ``out_dtype``."""
+    """out[row, h] = sum_g mix[h, g] o[row, g, kv(h)] for ``o`` [rows, heads_q, heads_kv, v_dim], float32 or
+    bfloat16 (``mix`` None: the identity); [rows, heads_q * v_dim] in ``out_dtype``."""
     _dev(o, mix)
-    if o.dtype != torch.float32 or o.dim() != 4:
-        raise KernelLibraryError("the heads' results must be float32 [rows, heads_q, heads_kv, v_dim]")
+    if o.dim() != 4:
+        raise KernelLibraryError("the heads' results must be [rows, heads_q, heads_kv, v_dim]")
     n, hq, hkv, vd = o.shape
     if mix is not None and tuple(mix.shape) != (hq, hq):
         raise KernelLibraryError(f"the heads' mixing matrix must be [{hq}, {hq}]")
     out = torch.empty((n, hq * vd), dtype=out_dtype, device=o.device)
-    check(library.core().sb_head_mix(_p(out), _dt(out), _p(o), _p(mix), _dt(mix) if mix is not None else 0, n, hq, hkv, vd,
-                                     _stream()))
+    check(library.core().sb_head_mix(_p(out), _dt(out), _p(o), _dt(o), _p(mix), _dt(mix) if mix is not None else 0, n, hq, hkv,
+                                     vd, _stream()))
+    return out
+
+
+def shared_attention_mfma_ok(q_dtype, cache_dtype, head_dim: int, v_dim: int) -> bool:
+    return capped_attention_mfma_ok(q_dtype, cache_dtype, head_dim, v_dim)
+
+
+def attention_shared_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor,
+                          row_pos: torch.Tensor, tiles: torch.Tensor, heads_q: int, heads_kv: int, head_dim: int, v_dim: int,
+                          scale: float, r1: Optional[torch.Tensor], r2: Optional[torch.Tensor],
+                          chunks: Optional[int] = None) -> torch.Tensor:
+    """The matrix-core form of :func:`attention_shared_plain` (the kernels of :func:`attention_capped_mfma`
+    with the distance bias and every kv head's values): bfloat16 [rows, heads_q, heads_kv, v_dim].
+    ``tiles`` int32 [n, 4]: the rows in runs of up to 16 consecutive rows of one sequence."""
+    _dev(q, k_cache, v_cache, page_table, row_pos, tiles, r1, r2)
+    n = q.shape[0]
+    if q.dim() != 2 or q.shape[1] != heads_q * head_dim or q.dtype != torch.bfloat16:
+        raise KernelLibraryError(f"queries must be bfloat16 [rows, {heads_q * head_dim}]")
+    _check_cache_kv(k_cache, v_cache, heads_kv, head_dim, v_dim)
+    if k_cache.dtype != torch.bfloat16:
+        raise KernelLibraryError("the matrix-core kernel reads a bfloat16 cache")
+    _i32(row_pos, n, "row positions")
+    if page_table.dtype != torch.int32 or page_table.dim() != 2:
+        raise KernelLibraryError("page table must be int32 [sequences, pages]")
+    if tiles.dtype != torch.int32 or tiles.dim() != 2 or tiles.shape[1] != 4:
+        raise KernelLibraryError("row tiles must be int32 [n, 4]")
+    if (r1 is None) != (r2 is None):
+        raise KernelLibraryError("the distance bias needs both of its numbers a head")
+    if r1 is not None:
+        _f32_vec(r1, heads_q, "r1")
+        _f32_vec(r2, heads_q, "r2")
+    n_tiles, max_pages = tiles.shape[0], page_table.shape[1]
+    group = heads_q // heads_kv
+    blocks = max(1, n_tiles * heads_kv * heads_kv * ((group + 3) // 4))
+    if chunks is None:
+        chunks = max(1, min(max_pages, CAPPED_SPLIT_BLOCKS // blocks))
+    chunk_pages = (max_pages + chunks - 1) // chunks
+    chunks = (max_pages + chunk_pages - 1) // chunk_pages
+    part_o = part_ml = None
+    if chunks > 1:
+        part_o = torch.empty((chunks, n, heads_q * heads_kv, v_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((chunks, n, heads_q * heads_kv, 2), dtype=torch.float32, device=q.device)
+    out = torch.empty((n, heads_q, heads_kv, v_dim), dtype=torch.bfloat16, device=q.device)
+    lib = library.capped_attention_library(head_dim, v_dim)
+    check(lib.sb_cattn_shared_bf16(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(page_table), max_pages, k_cache.shape[0],
+                                   _p(row_pos), _p(tiles), n_tiles, n, heads_q, heads_kv, float(scale), 0, 0.0, 0, chunks,
+                                   chunk_pages, _p(part_o), _p(part_ml), _p(r1), _p(r2), 1, _stream()),
+          lib, "sb_cattn_last_error")
     return out
 
 
@@ -1636,7 +1684,12 @@ def attention_shared(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                      fast: bool = True) -> torch.Tensor:
     """Attention of a step's rows over the cache with a distance bias and the heads' weights mixed by
     ``mix`` [heads_q, heads_q]: every query head's weights against every key/value head's values, then the
-    mix of the results; [rows, heads_q * v_dim] in ``out_dtype``."""
-    o = attention_shared_plain(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_seq, heads_q, heads_kv, head_dim,
-                               v_dim, scale, r1, r2)
+    mix of the results; [rows, heads_q * v_dim] in ``out_dtype``.  bfloat16 with head sizes in steps of 16
+    runs on the matrix cores; everything else takes the plain kernel."""
+    if fast and shared_attention_mfma_ok(q.dtype, k_cache.dtype, head_dim, v_dim):
+        o = attention_shared_mfma(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_tiles(CAPPED_ROW_TILE), heads_q,
+                                  heads_kv, head_dim, v_dim, scale, r1, r2)
+    else:
+        o = attention_shared_plain(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_seq, heads_q, heads_kv, head_dim,
+                                   v_dim, scale, r1, r2)
     return head_mix(o, mix, out_dtype)

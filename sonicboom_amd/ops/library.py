@@ -79,7 +79,7 @@ _CORE_SIGNATURES = {
     "sb_delta_scan": [_P, _I, _I, _P, _I, _P, _I, _P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P],
     "sb_qk_rownorm_store": [_P, _I, _P, _I, _P, _P, _I, _F, _F, _I, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "sb_attention_shared": [_P, _P, _I, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _P, _P, _P],
-    "sb_head_mix": [_P, _I, _P, _P, _I, _I, _I, _I, _I, _P],
+    "sb_head_mix": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],
     "sb_latent_attention_bf16": [_P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _P, _P, _I, _P],
 }
 # Entry points of later kernels; declared when the library has them.
@@ -118,6 +118,8 @@ _CAPPED_ATTN_SIGNATURES = {
     # out, q, k_cache, v_cache, page_table, max_pages, n_pages, row_pos, tiles, n_tiles, n_rows, heads_q, heads_kv,
     # scale, window, softcap, sink, chunks, chunk_pages, part_o, part_ml, stream
     "sb_cattn_bf16": [_P, _P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _F, _I, _I, _I, _P, _P, _P],
+    # the same, then dist_r1, dist_r2, all_values, stream
+    "sb_cattn_shared_bf16": [_P, _P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _F, _I, _I, _I, _P, _P, _P, _P, _I, _P],
     "sb_cattn_tile_rows": [],
     "sb_cattn_key_dim": [],
     "sb_cattn_value_dim": [],

@@ -60,6 +60,8 @@ def shared_attention_spec(prefix: str, width: int, heads_q: int, heads_kv: int, 
 
 @register_part("mixer", "shared_attention")
 class SharedAttention(Mixer):
+    # a step's context lists its rows in runs of this many for the matrix-core kernel
+    row_tile = ops.CAPPED_ROW_TILE
     fuses_norm = True
     graph_safe = True     # its launches depend on device buffers only
 

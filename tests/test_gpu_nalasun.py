@@ -407,13 +407,14 @@ class Harness:
     """A cache and per-sequence states for one part alone, and ``feed``: rows of sequences in cuts through
     ``fn(h, x, ctx, binding)``, which adds into the float32 rows ``x`` that come back."""
 
-    def __init__(self, rt, cache_spec=None, states=None, width=64, pages=24, max_slots=4):
+    def __init__(self, rt, cache_spec=None, states=None, width=64, pages=24, max_slots=4, tiles=()):
         from sonicboom_amd.cache import PagedCache, group_entries
         self.rt, self.width = rt, width
         groups = group_entries({0: cache_spec.key()}) if cache_spec is not None else []
         shapes = {(0, name): (tuple(s.shape), s.dtype) for name, s in (states or {}).items()}
         self.cache = PagedCache(groups, 64 * pages, rt.cache_dtype, rt.device, shapes, max_slots=max_slots)
         self.has_cache = cache_spec is not None
+        self.tiles = (tiles,) if isinstance(tiles, int) else tuple(tiles or ())
 
     def binding(self):
         from sonicboom_amd.engine.model import LayerBinding
@@ -432,7 +433,7 @@ class Harness:
         try:
             for n in cuts:
                 self.cache.reserve([slot], [n])
-                ctx = StepContext(self.cache, [StepEntry(slot, [0] * n, ())], self.rt.device, ())
+                ctx = StepContext(self.cache, [StepEntry(slot, [0] * n, ())], self.rt.device, self.tiles)
                 ctx.shared = {}
                 x = torch.zeros((n, self.width), dtype=F32, device=DEV)
                 fn(h_rows[at:at + n].to(DEV).contiguous(), x, ctx, self.binding())
@@ -451,7 +452,7 @@ class Harness:
         try:
             lens = [s.shape[0] for s in seqs]
             self.cache.reserve(slots, lens)
-            ctx = StepContext(self.cache, [StepEntry(s, [0] * n, ()) for s, n in zip(slots, lens)], self.rt.device, ())
+            ctx = StepContext(self.cache, [StepEntry(s, [0] * n, ()) for s, n in zip(slots, lens)], self.rt.device, self.tiles)
             ctx.shared = {}
             x = torch.zeros((sum(lens), self.width), dtype=F32, device=DEV)
             fn(torch.cat(seqs).to(DEV).contiguous(), x, ctx, self.binding())
@@ -504,7 +505,8 @@ def mixer_of(spec, dtype, seed=0, scale=0.5, fast=True, edit=None):
 
 def mixer_harness(mixer, rt, width=64):
     ss = mixer.state_spec()
-    return Harness(rt, cache_spec=mixer.cache_spec(), states=ss if isinstance(ss, dict) else None, width=width)
+    return Harness(rt, cache_spec=mixer.cache_spec(), states=ss if isinstance(ss, dict) else None, width=width,
+                   tiles=getattr(mixer, "row_tile", None))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
