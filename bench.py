@@ -722,7 +722,7 @@ class AllOpsTimer:
             "attention_tall_ok", "attention_mfma_ok", "attention_decode_rope_ok", "gate_code", "reduce_resid_norm_ok",
             "attention_decode_pages_per_wave", "gemm_tile_shape", "gemm_few_rows_kernel", "mingru_chunk_rows",
             "loaded_paths", "check", "latent_attention_mfma_ok", "capped_attention_mfma_ok", "moe_max_top", "moe_plan",
-            "time_conv_max_taps", "state_scan_limits", "shared_attention_mfma_ok")
+            "time_conv_max_taps", "state_scan_limits", "state_scan_chunk_rows", "shared_attention_mfma_ok")
     INNER = ("attention_plain", "attention_decode_mfma", "attention_prefill_mfma", "latent_attention_plain",
              "latent_attention_mfma", "attention_capped_plain", "attention_capped_mfma",
              "moe_product_plain", "attention_shared_plain", "attention_shared_mfma",

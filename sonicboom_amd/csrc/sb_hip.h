@@ -331,18 +331,25 @@ int sb_time_conv_keep(const void *in, int in_dtype, int in_stride, float *state,
  * sb_delta_scan: q, k (of head a / (heads / kv_heads)) to unit vectors (eps_unit inside the root), q times
  *   D^-1/2; beta = sigmoid(b); g = exp(-exp(a_log[a]) softplus(decay + dt_bias)) per key channel;
  *   S = g S; u = beta (v - S^T k); S += k u^T; o = S^T q; out = o / sqrt(mean(o^2) + eps) w sigmoid(gate).
- *   qkv rows hold q [kv_heads D] | k [kv_heads D] | v [heads E]. */
+ *   qkv rows hold q [kv_heads D] | k [kv_heads D] | v [heads E].
+ * With chunks (int32 [n_chunks, 4]: first row, rows <= chunk_rows, sequence, 0; sequence after sequence in row
+ * order, each sequence's runs full but its last) both take the chunked form in three launches: every chunk from an
+ * empty matrix, the chunks' results carried along each sequence, every chunk again from the matrix that comes in.
+ * Scratch, float32: part [n_chunks, heads, N, P] and part_decay [n_chunks, heads] for sb_ssd_scan,
+ * part [n_chunks, heads, D * E + D * D] for sb_delta_scan. */
 int sb_state_scan_max_rows(void);
 int sb_state_scan_max_cols(void);
+int sb_state_scan_chunk_rows(void);
 int sb_ssd_scan(float *out, int out_stride, const float *z, int z_stride, const float *x, int x_stride, const float *bc,
                 int bc_stride, int c_off, const float *dt, int dt_stride, const float *dt_bias, const float *a_log,
                 const float *d_skip, float *state, const int32_t *cu_rows, const int32_t *slots, int n_seqs, int heads,
-                int groups, int N, int P, void *stream);
+                int groups, int N, int P, const int32_t *chunks, int n_chunks, int chunk_rows, float *part, float *part_decay,
+                void *stream);
 int sb_delta_scan(void *out, int out_dtype, int out_stride, const float *qkv, int qkv_stride, const float *beta,
                   int beta_stride, const float *decay, int decay_stride, const float *gate, int gate_stride,
                   const float *dt_bias, const float *a_log, const void *w, int w_dtype, float *state,
                   const int32_t *cu_rows, const int32_t *slots, int n_seqs, int heads, int kv_heads, int D, int E,
-                  float eps, float eps_unit, void *stream);
+                  float eps, float eps_unit, const int32_t *chunks, int n_chunks, int chunk_rows, float *part, void *stream);
 
 /* Attention whose heads share their weights.
  * sb_qk_rownorm_store: from f32 rows [q: heads_q dk | k: heads_kv dk]: q / rms(q, the whole part) * q_w *

@@ -1503,13 +1503,29 @@ def state_scan_limits():
     return int(lib.sb_state_scan_max_rows()), int(lib.sb_state_scan_max_cols())
 
 
+def state_scan_chunk_rows() -> int:
+    """The rows of a chunk of the chunked forms of :func:`ssd_scan` and :func:`delta_scan`."""
+    return int(library.core().sb_state_scan_chunk_rows())
+
+
+def _scan_chunks(chunks: Optional[torch.Tensor]) -> int:
+    if chunks is None:
+        return 0
+    _dev(chunks)
+    if chunks.dtype != torch.int32 or chunks.dim() != 2 or chunks.shape[1] != 4 or not chunks.is_contiguous() or not len(chunks):
+        raise KernelLibraryError("chunks must be int32 [n, 4] with a run at least")
+    return int(chunks.shape[0])
+
+
 def ssd_scan(z: torch.Tensor, x: torch.Tensor, b: torch.Tensor, c: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor,
              a_log: torch.Tensor, d_skip: torch.Tensor, state: torch.Tensor, ctx, heads: int, groups: int, n_state: int,
-             v_dim: int) -> torch.Tensor:
+             v_dim: int, chunks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The selective state-space recurrence over the rows of the step (see csrc/state_space.hip):
     ``z``, ``x`` [n, heads * v_dim], ``b``, ``c`` [n, groups * n_state] (column ranges of one tensor),
     ``dt`` [n, heads] before bias and softplus, all float32 (views of wider rows allowed);
-    ``state`` float32 [slots, heads, n_state, v_dim], moved on.  Returns y * silu(z), float32 [n, heads * v_dim]."""
+    ``state`` float32 [slots, heads, n_state, v_dim], moved on.  Returns y * silu(z), float32 [n, heads * v_dim].
+    ``chunks`` (int32 [m, 4], the step's rows in runs of at most :func:`state_scan_chunk_rows` rows of one
+    sequence, as the context lists them): the chunked form, for long prompts."""
     n = ctx.n_rows
     inner = heads * v_dim
     _f32_rows(z, n, inner, "z")
@@ -1525,20 +1541,25 @@ def ssd_scan(z: torch.Tensor, x: torch.Tensor, b: torch.Tensor, c: torch.Tensor,
         raise KernelLibraryError(f"the state must be float32 [slots, {heads}, {n_state}, {v_dim}]")
     out = torch.empty((n, inner), dtype=torch.float32, device=z.device)
     c_off = (c.data_ptr() - b.data_ptr()) // 4
+    m = _scan_chunks(chunks)
+    part = torch.empty((m, heads, n_state, v_dim), dtype=torch.float32, device=z.device) if m else None
+    part_decay = torch.empty((m, heads), dtype=torch.float32, device=z.device) if m else None
     check(library.core().sb_ssd_scan(_p(out), inner, _p(z), z.stride(0), _p(x), x.stride(0), _p(b), b.stride(0), c_off,
                                      _p(dt), dt.stride(0), _p(dt_bias), _p(a_log), _p(d_skip), _p(state), _p(ctx.cu_rows),
-                                     _p(ctx.slots), ctx.n_seqs, heads, groups, n_state, v_dim, _stream()))
+                                     _p(ctx.slots), ctx.n_seqs, heads, groups, n_state, v_dim, _p(chunks), m,
+                                     state_scan_chunk_rows() if m else 0, _p(part), _p(part_decay), _stream()))
     return out
 
 
 def delta_scan(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, gate: torch.Tensor, dt_bias: torch.Tensor,
                a_log: torch.Tensor, weight: torch.Tensor, state: torch.Tensor, ctx, heads: int, kv_heads: int, dim: int,
-               v_dim: int, eps: float, eps_unit: float, out_dtype: torch.dtype) -> torch.Tensor:
+               v_dim: int, eps: float, eps_unit: float, out_dtype: torch.dtype,
+               chunks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The delta rule with a decay per key channel over the rows of the step (see csrc/state_space.hip):
     ``qkv`` [n, 2 * kv_heads * dim + heads * v_dim] after the short convolution, ``beta`` [n, heads],
     ``decay`` [n, heads * dim], ``gate`` [n, heads * v_dim] before their activations, all float32;
     ``state`` float32 [slots, heads, dim, v_dim], moved on.  Returns the normed, gated heads
-    [n, heads * v_dim] in ``out_dtype``."""
+    [n, heads * v_dim] in ``out_dtype``.  ``chunks``: as for :func:`ssd_scan`."""
     n = ctx.n_rows
     _f32_rows(qkv, n, 2 * kv_heads * dim + heads * v_dim, "q, k and v")
     _f32_rows(beta, n, heads, "beta")
@@ -1552,10 +1573,13 @@ def delta_scan(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, gate:
     if state.dtype != torch.float32 or tuple(state.shape[1:]) != (heads, dim, v_dim) or not state.is_contiguous():
         raise KernelLibraryError(f"the state must be float32 [slots, {heads}, {dim}, {v_dim}]")
     out = torch.empty((n, heads * v_dim), dtype=out_dtype, device=qkv.device)
+    m = _scan_chunks(chunks)
+    part = torch.empty((m, heads, dim, v_dim + dim), dtype=torch.float32, device=qkv.device) if m else None
     check(library.core().sb_delta_scan(_p(out), _dt(out), heads * v_dim, _p(qkv), qkv.stride(0), _p(beta), beta.stride(0),
                                        _p(decay), decay.stride(0), _p(gate), gate.stride(0), _p(dt_bias), _p(a_log),
                                        _p(weight), _dt(weight), _p(state), _p(ctx.cu_rows), _p(ctx.slots), ctx.n_seqs, heads,
-                                       kv_heads, dim, v_dim, float(eps), float(eps_unit), _stream()))
+                                       kv_heads, dim, v_dim, float(eps), float(eps_unit), _p(chunks), m,
+                                       state_scan_chunk_rows() if m else 0, _p(part), _stream()))
     return out
 
 

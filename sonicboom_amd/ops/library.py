@@ -75,8 +75,11 @@ _CORE_SIGNATURES = {
     "sb_time_conv_keep": [_P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _P],
     "sb_state_scan_max_rows": [],
     "sb_state_scan_max_cols": [],
-    "sb_ssd_scan": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
-    "sb_delta_scan": [_P, _I, _I, _P, _I, _P, _I, _P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P],
+    "sb_state_scan_chunk_rows": [],
+    "sb_ssd_scan": [_P, _I, _P, _I, _P, _I, _P, _I, _I, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _I, _I, _P, _P,
+                    _P],
+    "sb_delta_scan": [_P, _I, _I, _P, _I, _P, _I, _P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _F, _P, _I,
+                      _I, _P, _P],
     "sb_qk_rownorm_store": [_P, _I, _P, _I, _P, _P, _I, _F, _F, _I, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "sb_attention_shared": [_P, _P, _I, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _P, _P, _P],
     "sb_head_mix": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _P],

@@ -25,6 +25,11 @@ and the scan kernels take softplus, exponentials, sigmoids, unit vectors and the
 there.  The matrices and the convolutions' last inputs are per-sequence state of the cache (a row per
 slot, zeroed when the slot is handed out, moved on by every step), so prompts cut into steps,
 batches and decoding all run the same recurrence, to the bit in the 32-bit path.
+
+With bfloat16 activations a step that brings a sequence more than two chunks of rows takes the
+scans' chunked form (every chunk from an empty matrix, the results carried along the sequence, every
+chunk again from the matrix that comes in; float32 throughout), which spreads a long prompt over
+the whole chip; it differs from the walk by rounding.  The 32-bit path always walks.
 """
 from __future__ import annotations
 
@@ -46,6 +51,15 @@ DELTA_NAMES = {"q": "q", "k": "k", "v": "v", "q_conv": "q.conv", "k_conv": "k.co
 
 def _vec(t: torch.Tensor) -> torch.Tensor:
     return t.float().contiguous()
+
+
+def _chunk_rows(rt, tensor: torch.Tensor) -> int:
+    """The chunk of the scans' chunked form, 0 where the mixer always walks."""
+    return ops.state_scan_chunk_rows() if rt.act_dtype != torch.float32 and tensor.is_cuda else 0
+
+
+def _chunks(chunk: int, ctx):
+    return ctx.row_tiles(chunk) if chunk and ctx.max_new > 2 * chunk else None
 
 
 def _check_taps(taps: int) -> None:
@@ -97,6 +111,8 @@ class SSD(Mixer):
         self.dt_bias, self.a_log, self.d_skip = _vec(tensors["dt_bias"]), _vec(tensors["a_log"]), _vec(tensors["d_skip"])
         self.norm = tensors["norm"].contiguous()
         self.out = Linear(tensors["out"], None, rt.fast_kernels)
+        self.chunk = _chunk_rows(rt, self.norm)
+        self.row_tile = self.chunk or None
 
     def state_spec(self):
         return {"conv": StateSpec((self.taps - 1, self.inner + 2 * self.bc), torch.float32),
@@ -109,7 +125,7 @@ class SSD(Mixer):
                             columns=(inner, inner + 2 * bc))
         y = ops.ssd_scan(proj[:, :inner], xbc[:, :inner], xbc[:, inner:inner + bc], xbc[:, inner + bc:],
                          proj[:, 2 * inner + 2 * bc:], self.dt_bias, self.a_log, self.d_skip, binding.states["matrix"], ctx,
-                         self.heads, self.groups, self.n_state, self.v_dim)
+                         self.heads, self.groups, self.n_state, self.v_dim, _chunks(self.chunk, ctx))
         y = ops.rmsnorm(y, self.norm, self.eps, self.rt.act_dtype, groups=self.norm_groups)
         return self.out.add_into(y, x, then_norm, self.rt.act_dtype, scale=self.out_scale)
 
@@ -173,6 +189,8 @@ class ChannelDelta(Mixer):
         self.dt_bias, self.a_log = _vec(tensors["dt_bias"]), _vec(tensors["a_log"])
         self.norm = tensors["norm"].contiguous()
         self.out = Linear(tensors["out"], None, rt.fast_kernels)
+        self.chunk = _chunk_rows(rt, self.norm)
+        self.row_tile = self.chunk or None
 
     def state_spec(self):
         return {"conv": StateSpec((self.taps - 1, self.qkv_width), torch.float32),
@@ -187,5 +205,5 @@ class ChannelDelta(Mixer):
         gate = self.gate_up(self.gate_down(h, act), torch.float32)
         y = ops.delta_scan(qkv, proj[:, self.qkv_width:], decay, gate, self.dt_bias, self.a_log, self.norm,
                            binding.states["matrix"], ctx, self.heads, self.kv_heads, self.head_dim, self.v_dim, self.eps,
-                           UNIT_EPS, act)
+                           UNIT_EPS, act, _chunks(self.chunk, ctx))
         return self.out.add_into(y, x, then_norm, act, scale=self.out_scale)

@@ -731,3 +731,62 @@ def test_the_router_kernel_scores_like_the_plain_one():
         chosen, weight = N.route(z.numpy().astype(np.float64), top, 1.5)
         assert np.array_equal(ids.cpu().numpy(), chosen)
         assert np.allclose(w[:, :top].cpu().numpy(), weight, atol=1e-6)
+
+
+# ---- the scans' chunked form against the walk ------------------------------------------------------------------
+
+
+def scan_context(lens, slots, chunk):
+    """What the scans read of a step: rows of sequences of ``lens`` rows in state rows ``slots``, and its chunks."""
+    from types import SimpleNamespace
+    from sonicboom_amd.engine.step import row_runs
+    cu = np.zeros(len(lens) + 1, dtype=np.int32)
+    cu[1:] = np.cumsum(lens)
+    i32 = lambda a: torch.tensor(np.asarray(a, dtype=np.int32), device=DEV)
+    return SimpleNamespace(n_rows=int(cu[-1]), n_seqs=len(lens), cu_rows=i32(cu), slots=i32(slots)), i32(row_runs(lens, cu, chunk))
+
+
+SCAN_LENS = ([200], [64], [65, 1, 128, 7], [3, 129, 300])
+
+
+@pytest.mark.parametrize("lens", SCAN_LENS)
+@pytest.mark.parametrize("heads, groups, state, vdim", [(4, 2, 16, 32), (3, 1, 24, 20), (2, 2, 128, 64), (1, 1, 7, 130)])
+def test_state_space_scan_in_chunks_equals_the_walk(lens, heads, groups, state, vdim):
+    from sonicboom_amd import ops
+    chunk = ops.state_scan_chunk_rows()
+    slots = [5, 0, 3, 2][:len(lens)]
+    ctx, chunks = scan_context(lens, slots, chunk)
+    n, inner, bc = ctx.n_rows, heads * vdim, groups * state
+    rows = rand(n, 2 * inner + 2 * bc + heads, seed=31).to(DEV)
+    z, x, b, c, dt = rows[:, :inner], rows[:, inner:2 * inner], rows[:, 2 * inner:2 * inner + bc], \
+        rows[:, 2 * inner + bc:2 * inner + 2 * bc], rows[:, 2 * inner + 2 * bc:]
+    vecs = [rand(heads, scale=0.5, seed=32 + i).to(DEV) for i in range(3)]
+    start = rand(6, heads, state, vdim, seed=35).to(DEV)
+    walked, chunked = start.clone(), start.clone()
+    want = ops.ssd_scan(z, x, b, c, dt, *vecs, walked, ctx, heads, groups, state, vdim)
+    got = ops.ssd_scan(z, x, b, c, dt, *vecs, chunked, ctx, heads, groups, state, vdim, chunks)
+    part_close(got, want.cpu().numpy(), "float32", "the state space's outputs in chunks", f32=2e-5)
+    part_close(chunked, walked.cpu().numpy(), "float32", "the state space's states after chunks", f32=2e-5)
+    assert torch.equal(chunked[1], start[1]) and torch.equal(chunked[4], start[4]), "a state row of no sequence was written"
+
+
+@pytest.mark.parametrize("lens", SCAN_LENS)
+@pytest.mark.parametrize("heads, kv_heads, dim, vdim", [(4, 2, 16, 32), (3, 1, 12, 20), (2, 2, 128, 128), (1, 1, 70, 9), (2, 1, 8, 200)])
+def test_delta_rule_scan_in_chunks_equals_the_walk(lens, heads, kv_heads, dim, vdim):
+    from sonicboom_amd import ops
+    chunk = ops.state_scan_chunk_rows()
+    slots = [5, 0, 3, 2][:len(lens)]
+    ctx, chunks = scan_context(lens, slots, chunk)
+    n = ctx.n_rows
+    qkv = rand(n, 2 * kv_heads * dim + heads * vdim, seed=41).to(DEV)
+    beta, decay, gate = rand(n, heads, seed=42).to(DEV), rand(n, heads * dim, seed=43).to(DEV), rand(n, heads * vdim, seed=44).to(DEV)
+    dt_bias, a_log, w = rand(heads * dim, scale=0.5, seed=45).to(DEV), (rand(heads, scale=0.5, seed=46) - 1.0).to(DEV), \
+        (1.0 + rand(vdim, scale=0.1, seed=47)).to(DEV)
+    start = rand(6, heads, dim, vdim, seed=48).to(DEV)
+    walked, chunked = start.clone(), start.clone()
+    args = (heads, kv_heads, dim, vdim, 1e-5, 1e-6, F32)
+    want = ops.delta_scan(qkv, beta, decay, gate, dt_bias, a_log, w, walked, ctx, *args)
+    got = ops.delta_scan(qkv, beta, decay, gate, dt_bias, a_log, w, chunked, ctx, *args, chunks)
+    part_close(got, want.cpu().numpy(), "float32", "the delta rule's outputs in chunks", f32=5e-5)
+    part_close(chunked, walked.cpu().numpy(), "float32", "the delta rule's states after chunks", f32=5e-5)
+    assert torch.equal(chunked[1], start[1]) and torch.equal(chunked[4], start[4]), "a state row of no sequence was written"
