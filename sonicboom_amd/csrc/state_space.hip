@@ -36,7 +36,7 @@ namespace {
 
 constexpr int RB = 8;          // rows staged in LDS at a time
 constexpr int CB = 2;          // columns of S a thread holds
-constexpr int CARRY_COLS = 16; // value columns a block of the delta rule's carry moves on
+constexpr int CARRY_COLS = 4;  // value columns a block of the delta rule's carry moves on
 enum { WHOLE = 0, LOCAL = 1, FROM = 2 };
 
 __device__ __forceinline__ float softplus_f(float a) { return a > 20.0f ? a : log1pf(expf(a)); }
@@ -407,7 +407,6 @@ __global__ void __launch_bounds__(256) delta_carry_kernel(DeltaArgs a, int chunk
   for (int c = 0; c < n; ++c) {
     float *base = a.part + (size_t(c0 + c) * a.heads + head) * part_size;
     float *pp = base + size_t(d) * a.E + e0;
-    const float *mt = base + size_t(a.D) * a.E + d;
     float acc[CPT];
 #pragma unroll
     for (int j = 0; j < CPT; ++j) acc[j] = (row_live && e0 + j < a.E) ? pp[j] : 0.0f;
@@ -419,10 +418,16 @@ __global__ void __launch_bounds__(256) delta_carry_kernel(DeltaArgs a, int chunk
 #pragma unroll
       for (int j = 0; j < CPT; ++j)
         if (e0 + j < a.E) pp[j] = cur[j];
-      for (int k0 = 0; k0 < a.D; k0 += 32) {          // 32 numbers of M_c a thread in flight
+      const float *mrow = base + size_t(a.D) * a.E;     // row k of M_c transposed, the same for every thread
+      for (int k0 = 0; k0 < a.D; k0 += 32) {            // 32 numbers of M_c a thread in flight
         float mv[32];
+        if (k0 + 32 <= a.D) {
 #pragma unroll
-        for (int u = 0; u < 32; ++u) mv[u] = k0 + u < a.D ? mt[size_t(k0 + u) * a.D] : 0.0f;
+          for (int u = 0; u < 32; ++u) { mv[u] = mrow[d]; mrow += a.D; }
+        } else {
+#pragma unroll
+          for (int u = 0; u < 32; ++u) { mv[u] = k0 + u < a.D ? mrow[d] : 0.0f; mrow += a.D; }
+        }
 #pragma unroll
         for (int u = 0; u < 32; ++u)
 #pragma unroll
