@@ -751,7 +751,7 @@ SCAN_LENS = ([200], [64], [65, 1, 128, 7], [3, 129, 300])
 
 @pytest.mark.parametrize("lens", SCAN_LENS)
 @pytest.mark.parametrize("heads, groups, state, vdim", [(4, 2, 16, 32), (3, 1, 24, 20), (2, 2, 128, 64), (1, 1, 7, 130), (2, 1, 160, 24),
-                                                        (1, 1, 40, 7)])
+                                                        (1, 1, 40, 7), (1, 1, 136, 140), (2, 2, 130, 100)])
 def test_state_space_scan_in_chunks_equals_the_walk(lens, heads, groups, state, vdim):
     from sonicboom_amd import ops
     chunk = ops.state_scan_chunk_rows()
@@ -773,7 +773,8 @@ def test_state_space_scan_in_chunks_equals_the_walk(lens, heads, groups, state, 
 
 @pytest.mark.parametrize("lens", SCAN_LENS)
 @pytest.mark.parametrize("heads, kv_heads, dim, vdim", [(4, 2, 16, 32), (3, 1, 12, 20), (2, 2, 128, 128), (1, 1, 70, 9), (2, 1, 8, 200),
-                                                          (2, 1, 144, 40), (1, 1, 33, 255)])
+                                                          (2, 1, 144, 40), (1, 1, 33, 255), (1, 1, 136, 140),
+                                                          (2, 2, 130, 100)])
 def test_delta_rule_scan_in_chunks_equals_the_walk(lens, heads, kv_heads, dim, vdim):
     from sonicboom_amd import ops
     chunk = ops.state_scan_chunk_rows()
