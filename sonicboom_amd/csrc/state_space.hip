@@ -77,13 +77,16 @@ struct SsdArgs {
   const int32_t *chunks;                 // [n_chunks, 4]: first row, rows, sequence, 0
   float *part;                           // [n_chunks, heads, N, P]: A_c, then S_in(c)
   float *part_decay;                     // [n_chunks, heads]: the logarithm of the chunk's product of decays
+  int vec4;                              // B and C of a row can be read four numbers at a time
 };
 
 // A thread holds NMAX / SPLIT rows of CB adjacent columns of S; SPLIT adjacent lanes share the columns.
 template <int NMAX, int SPLIT, int MODE>
 __global__ void __launch_bounds__(256) ssd_scan_kernel(SsdArgs a) {
   constexpr int NT = NMAX / SPLIT;
-  __shared__ float bs[RB][NMAX + 4 * SPLIT], cs[RB][NMAX + 4 * SPLIT], xs[RB][256], zs[RB][256], dts[RB], decs[RB];
+  // xs holds a row's x until the row is walked and its y (with the skip) from then on
+  __shared__ __attribute__((aligned(16))) float bs[RB][NMAX + 4 * SPLIT], cs[RB][NMAX + 4 * SPLIT];
+  __shared__ float xs[RB][256], zs[RB][256], dts[RB], decs[RB], logs[RB];
   const int head = blockIdx.x, p0 = (threadIdx.x / SPLIT) * CB, n0 = (threadIdx.x % SPLIT) * NT;
   const int l0 = staged<NT>(n0);
   int seq, r0, r1;
@@ -108,30 +111,55 @@ __global__ void __launch_bounds__(256) ssd_scan_kernel(SsdArgs a) {
   for (int rb = r0; rb < r1; rb += RB) {
     const int nr = min(RB, r1 - rb);
     __syncthreads();
-    // B and C of the rows, four elements a thread in flight
-    for (int base = threadIdx.x; base < nr * NMAX; base += 4 * blockDim.x) {
-      float bv[4], cv[4];
+    if (a.vec4) {
+      // B and C of the rows, two loads of four numbers each a thread in flight
+      constexpr int QUADS = NMAX / 4;
+      for (int base = threadIdx.x; base < nr * QUADS; base += 2 * blockDim.x) {
+        float4 bv[2], cv[2];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int i = base + u * blockDim.x, row = i / NMAX, n = i % NMAX;
-        const bool ok = i < nr * NMAX && n < a.N;
-        const float *src = a.bc + size_t(rb + row) * a.bc_stride + g * a.N + n;
-        bv[u] = ok ? src[0] : 0.0f;
-        cv[u] = (MODE != LOCAL && ok) ? src[a.c_off] : 0.0f;
+        for (int u = 0; u < 2; ++u) {
+          const int i = base + u * blockDim.x, row = i / QUADS, n = (i % QUADS) * 4;
+          const bool ok = i < nr * QUADS && n < a.N;
+          const float *src = a.bc + size_t(rb + row) * a.bc_stride + g * a.N + n;
+          bv[u] = ok ? *(const float4 *)src : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+          cv[u] = (MODE != LOCAL && ok) ? *(const float4 *)(src + a.c_off) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int i = base + u * blockDim.x, row = i / QUADS, n = (i % QUADS) * 4;
+          if (i < nr * QUADS) {
+            *(float4 *)&bs[row][staged<NT>(n)] = bv[u];
+            if (MODE != LOCAL) *(float4 *)&cs[row][staged<NT>(n)] = cv[u];
+          }
+        }
       }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int i = base + u * blockDim.x, row = i / NMAX, n = i % NMAX;
-        if (i < nr * NMAX) {
-          bs[row][staged<NT>(n)] = bv[u];
-          if (MODE != LOCAL) cs[row][staged<NT>(n)] = cv[u];
+    } else {
+      // B and C of the rows, four elements a thread in flight
+      for (int base = threadIdx.x; base < nr * NMAX; base += 4 * blockDim.x) {
+        float bv[4], cv[4];
+  #pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = base + u * blockDim.x, row = i / NMAX, n = i % NMAX;
+          const bool ok = i < nr * NMAX && n < a.N;
+          const float *src = a.bc + size_t(rb + row) * a.bc_stride + g * a.N + n;
+          bv[u] = ok ? src[0] : 0.0f;
+          cv[u] = (MODE != LOCAL && ok) ? src[a.c_off] : 0.0f;
+        }
+  #pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = base + u * blockDim.x, row = i / NMAX, n = i % NMAX;
+          if (i < nr * NMAX) {
+            bs[row][staged<NT>(n)] = bv[u];
+            if (MODE != LOCAL) cs[row][staged<NT>(n)] = cv[u];
+          }
         }
       }
     }
     if (threadIdx.x < nr) {
       const float dt = softplus_f(a.dt[size_t(rb + threadIdx.x) * a.dt_stride + head] + bias);
       dts[threadIdx.x] = dt;
-      decs[threadIdx.x] = -rate * dt;
+      logs[threadIdx.x] = -rate * dt;
+      decs[threadIdx.x] = expf(-rate * dt);
     }
     if (n0 == 0) {
 #pragma unroll
@@ -147,8 +175,8 @@ __global__ void __launch_bounds__(256) ssd_scan_kernel(SsdArgs a) {
     __syncthreads();
 #pragma unroll 1
     for (int i = 0; i < nr; ++i) {
-      const float dt = dts[i], decay = expf(decs[i]);
-      if (MODE == LOCAL) log_decay += decs[i];
+      const float dt = dts[i], decay = decs[i];
+      if (MODE == LOCAL) log_decay += logs[i];
       float xv[CB], dx[CB], y[CB];
 #pragma unroll
       for (int c = 0; c < CB; ++c) { xv[c] = xs[i][p0 + c]; dx[c] = dt * xv[c]; y[c] = 0.0f; }
@@ -165,12 +193,18 @@ __global__ void __launch_bounds__(256) ssd_scan_kernel(SsdArgs a) {
 #pragma unroll
         for (int c = 0; c < CB; ++c) {
           const float yy = fmaf(skip, xv[c], lanes_sum<SPLIT>(y[c]));
-          if (n0 == 0 && p0 + c < a.P) {
-            const float zv = zs[i][p0 + c];
-            a.out[size_t(rb + i) * a.out_stride + head * a.P + p0 + c] = yy * (zv * sigmoid_f(zv));
-          }
+          if (n0 == 0) xs[i][p0 + c] = yy;         // the lanes that share the column have read x by now
         }
       }
+    }
+    if (MODE != LOCAL) {
+      // the gate and the store, an element a thread
+      __syncthreads();
+      for (int i = 0; i < nr; ++i)
+        for (int p = threadIdx.x; p < a.P; p += blockDim.x) {
+          const float zv = zs[i][p];
+          a.out[size_t(rb + i) * a.out_stride + head * a.P + p] = xs[i][p] * (zv * sigmoid_f(zv));
+        }
     }
   }
   if (MODE != FROM) {
@@ -505,7 +539,8 @@ extern "C" int sb_ssd_scan(float *out, int out_stride, const float *z, int z_str
   SB_SUPPORT(!chunks || n_chunks <= 65535, "sb_ssd_scan: more than 65535 chunks");
   if (n_seqs == 0) return SB_OK;
   SsdArgs a{out, out_stride, z, z_stride, x, x_stride, bc, bc_stride, c_off, dt, dt_stride, dt_bias, a_log, d_skip, state,
-            cu_rows, slots, heads, groups, N, P, chunks, part, part_decay};
+            cu_rows, slots, heads, groups, N, P, chunks, part, part_decay,
+            (N % 4 == 0 && bc_stride % 4 == 0 && c_off % 4 == 0 && (uintptr_t)bc % 16 == 0) ? 1 : 0};
   const int split = lanes_a_column(N, P);
   hipStream_t s = (hipStream_t)stream;
   if (!chunks) {
