@@ -256,6 +256,7 @@ struct DeltaArgs {
   float eps, eps_unit;
   const int32_t *chunks;                 // [n_chunks, 4]: first row, rows, sequence, 0
   float *part;                           // [n_chunks, heads, D * E + D * D]: A_c (then S_in(c)) [D, E] | M_c transposed [D, D]
+  int vec4;                              // q, k, the decays and their bias can be read four numbers at a time
 };
 
 // A thread holds DMAX / SPLIT rows of CB adjacent columns of S; SPLIT adjacent lanes share the columns.
@@ -264,7 +265,8 @@ struct DeltaArgs {
 template <int DMAX, int SPLIT, int MODE>
 __global__ void __launch_bounds__(256) delta_scan_kernel(DeltaArgs a) {
   constexpr int DT = DMAX / SPLIT;
-  __shared__ float qs[MODE == LOCAL ? 1 : RB][DMAX + 4 * SPLIT], ks[RB][DMAX + 4 * SPLIT], gs[RB][DMAX + 4 * SPLIT];
+  __shared__ __attribute__((aligned(16))) float qs[MODE == LOCAL ? 1 : RB][DMAX + 4 * SPLIT], ks[RB][DMAX + 4 * SPLIT],
+      gs[RB][DMAX + 4 * SPLIT];
   __shared__ float vs[RB][512], os[MODE == LOCAL ? 1 : RB][512], q_inv[RB], k_inv[RB], betas[RB], o_inv[RB];
   const int head = blockIdx.x;
   const int cl = (threadIdx.x / SPLIT) * CB, d0 = (threadIdx.x % SPLIT) * DT, l0 = staged<DT>(d0);
@@ -297,25 +299,49 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(DeltaArgs a) {
   for (int rb = r0; rb < r1; rb += RB) {
     const int nr = min(RB, r1 - rb);
     __syncthreads();
-    // the head's queries and keys as they came, and the decays of its key channels; four elements a thread in flight
-    for (int base = threadIdx.x; base < nr * DMAX; base += 4 * blockDim.x) {
-      float qv[4], kv[4], gv[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int i = base + u * blockDim.x, row = i / DMAX, d = i % DMAX;
-        const bool ok = i < nr * DMAX && d < a.D;
+    if (a.vec4) {
+      // the head's queries and keys as they came, and the decays of its key channels, four numbers a load
+      constexpr int QUADS = DMAX / 4;
+      for (int i = threadIdx.x; i < nr * QUADS; i += blockDim.x) {
+        const int row = i / QUADS, d = (i % QUADS) * 4;
+        const bool ok = d < a.D;
+        const float4 zero = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         const float *src = a.qkv + size_t(rb + row) * a.qkv_stride + kvh * a.D + d;
-        qv[u] = (MODE != LOCAL && ok) ? src[0] : 0.0f;
-        kv[u] = ok ? src[GD] : 0.0f;
-        gv[u] = ok ? a.decay[size_t(rb + row) * a.decay_stride + head * a.D + d] + a.dt_bias[head * a.D + d] : 0.0f;
+        const float4 qv = (MODE != LOCAL && ok) ? *(const float4 *)src : zero;
+        const float4 kv = ok ? *(const float4 *)(src + GD) : zero;
+        const float4 av = ok ? *(const float4 *)(a.decay + size_t(rb + row) * a.decay_stride + head * a.D + d) : zero;
+        const float4 bv = ok ? *(const float4 *)(a.dt_bias + head * a.D + d) : zero;
+        float4 gv = make_float4(1.0f, 1.0f, 1.0f, 1.0f);
+        if (ok) {
+          gv.x = expf(-rate * softplus_f(av.x + bv.x)); gv.y = expf(-rate * softplus_f(av.y + bv.y));
+          gv.z = expf(-rate * softplus_f(av.z + bv.z)); gv.w = expf(-rate * softplus_f(av.w + bv.w));
+        }
+        const int at = staged<DT>(d);
+        if (MODE != LOCAL) *(float4 *)&qs[row][at] = qv;
+        *(float4 *)&ks[row][at] = kv;
+        *(float4 *)&gs[row][at] = gv;
       }
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int i = base + u * blockDim.x, row = i / DMAX, d = i % DMAX;
-        if (i < nr * DMAX) {
-          if (MODE != LOCAL) qs[row][staged<DT>(d)] = qv[u];
-          ks[row][staged<DT>(d)] = kv[u];
-          gs[row][staged<DT>(d)] = d < a.D ? expf(-rate * softplus_f(gv[u])) : 1.0f;
+    } else {
+      // the head's queries and keys as they came, and the decays of its key channels; four elements a thread in flight
+      for (int base = threadIdx.x; base < nr * DMAX; base += 4 * blockDim.x) {
+        float qv[4], kv[4], gv[4];
+  #pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = base + u * blockDim.x, row = i / DMAX, d = i % DMAX;
+          const bool ok = i < nr * DMAX && d < a.D;
+          const float *src = a.qkv + size_t(rb + row) * a.qkv_stride + kvh * a.D + d;
+          qv[u] = (MODE != LOCAL && ok) ? src[0] : 0.0f;
+          kv[u] = ok ? src[GD] : 0.0f;
+          gv[u] = ok ? a.decay[size_t(rb + row) * a.decay_stride + head * a.D + d] + a.dt_bias[head * a.D + d] : 0.0f;
+        }
+  #pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = base + u * blockDim.x, row = i / DMAX, d = i % DMAX;
+          if (i < nr * DMAX) {
+            if (MODE != LOCAL) qs[row][staged<DT>(d)] = qv[u];
+            ks[row][staged<DT>(d)] = kv[u];
+            gs[row][staged<DT>(d)] = d < a.D ? expf(-rate * softplus_f(gv[u])) : 1.0f;
+          }
         }
       }
     }
@@ -387,20 +413,17 @@ __global__ void __launch_bounds__(256) delta_scan_kernel(DeltaArgs a) {
         if (lane == 0) o_inv[i] = 1.0f / sqrtf(sq / float(a.E) + a.eps);
       }
       __syncthreads();
-      if (d0 == 0) {
-#pragma unroll
-        for (int c = 0; c < CB; ++c) {
-          const int col = col0 + c;
-          if (col < a.E) {
-            const float wv = ld_dyn(a.w, a.w_dtype, col);
-            for (int i = 0; i < nr; ++i) {
-              const float gate = sigmoid_f(a.gate[size_t(rb + i) * a.gate_stride + head * a.E + col]);
-              const float y = ((os[i][cl + c] * o_inv[i]) * wv) * gate;
-              const size_t at = size_t(rb + i) * a.out_stride + head * a.E + col;
-              if (a.out_dtype == SB_F32) ((float *)a.out)[at] = y;
-              else ((bf16_t *)a.out)[at] = f32_to_bf16(y);
-            }
-          }
+      // norm's weight, gate and store, an element a thread
+      // (a block wider than the head takes several rows a pass)
+      const int pass = max(1, int(blockDim.x) / a.E), i0 = threadIdx.x / a.E;
+      for (int e = threadIdx.x - i0 * a.E; i0 < pass && e < a.E; e += blockDim.x) {
+        const float wv = ld_dyn(a.w, a.w_dtype, e);
+        for (int i = i0; i < nr; i += pass) {
+          const float gate = sigmoid_f(a.gate[size_t(rb + i) * a.gate_stride + head * a.E + e]);
+          const float y = ((os[i][e] * o_inv[i]) * wv) * gate;
+          const size_t at = size_t(rb + i) * a.out_stride + head * a.E + e;
+          if (a.out_dtype == SB_F32) ((float *)a.out)[at] = y;
+          else ((bf16_t *)a.out)[at] = f32_to_bf16(y);
         }
       }
     }
@@ -570,7 +593,9 @@ extern "C" int sb_delta_scan(void *out, int out_dtype, int out_stride, const flo
   SB_SUPPORT(!chunks || n_chunks <= 65535, "sb_delta_scan: more than 65535 chunks");
   if (n_seqs == 0) return SB_OK;
   DeltaArgs a{out, out_dtype, out_stride, qkv, qkv_stride, beta, beta_stride, decay, decay_stride, gate, gate_stride, dt_bias,
-              a_log, w, w_dtype, state, cu_rows, slots, heads, kv_heads, D, E, eps, eps_unit, chunks, part};
+              a_log, w, w_dtype, state, cu_rows, slots, heads, kv_heads, D, E, eps, eps_unit, chunks, part,
+              (D % 4 == 0 && qkv_stride % 4 == 0 && decay_stride % 4 == 0 && (uintptr_t)qkv % 16 == 0 && (uintptr_t)decay % 16 == 0 &&
+               (uintptr_t)dt_bias % 16 == 0) ? 1 : 0};
   const int split = lanes_a_column(D, E);
   const int threads = scan_threads(E, split);
   hipStream_t s = (hipStream_t)stream;
