@@ -13,9 +13,12 @@
 //     out_t = o_t / sqrt(mean(o_t^2) + eps) * w * sigmoid(gate_t)
 //   head a reads q and k of head a / (heads / kv_heads).
 //
-// Both walk rows in order, a thread a column of S, which stays in the thread's registers; eight rows
-// at a time are staged in LDS (keys, queries, decays, values), so a row costs no trip to memory of
-// its own.  The state of sequence s lies in state[slots[s]] and goes from step to step.
+// Both walk rows in order.  A thread holds up to 32 rows of two adjacent columns of S in registers, the
+// lanes that share the columns sit side by side and sum by shuffles; eight rows at a time are staged in
+// LDS (keys, queries, decays, values; each lane's share four floats further on, so that the lanes of a
+// column read different banks), so a row costs no trip to memory of its own, and what follows the
+// recurrence (gate, output norm, store) is done an element a thread after the eight rows.  The state of
+// sequence s lies in state[slots[s]] and goes from step to step.
 //
 // Two forms.  The walk (WHOLE): a block a (sequence, head) from the sequence's first row of the step
 // to its last.  Every number of a row is computed by the same operations in the same order whatever
