@@ -1,2 +1,2 @@
 """Built-in architectures; importing the package registers them."""
-from . import nalasun, qwen2, rasizen, tatelorn  # noqa: F401
+from . import fitatar, nalasun, qwen2, rasizen, tatelorn  # noqa: F401

@@ -67,6 +67,7 @@ struct Args {
   float scale, softcap; int window, sink, chunk_pages;
   const float *dist_r1, *dist_r2;      // [heads_q] or NULL: the bias by the distance's logarithm
   int all_values;                      // 1: blockIdx.y also counts the kv head whose values are read
+  const float *sink_scores;            // [heads_q] or NULL: the sink's score a head (NULL: 0)
   unsigned round_blocks;       // blocks the GPU takes one of per CU
 };
 
@@ -124,7 +125,8 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
 
   const float neg_inf = -__builtin_inff();
   const bool with_sink = a.sink && chunk == 0;
-  float m = with_sink ? 0.0f : neg_inf;
+  // (scores are kept times log2(e): so is the sink's)
+  float m = with_sink ? ((a.sink_scores && has_head) ? a.sink_scores[h] * kLog2e : 0.0f) : neg_inf;
   float l = (with_sink && g == 0) ? 1.0f : 0.0f;      // a lane's share of the column's sum
   floatx4_t o[DT];
 #pragma unroll
@@ -382,6 +384,13 @@ extern "C" int sb_cattn_bf16(void *out, const void *q, const void *k_cache, cons
                               nullptr, 0, stream);
 }
 
+extern "C" int sb_cattn_sink_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
+                                  const int32_t *page_table, int max_pages, int n_pages, const int32_t *row_pos,
+                                  const int32_t *tiles, int n_tiles, int n_rows, int heads_q, int heads_kv, float scale,
+                                  int window, float softcap, int sink, int chunks, int chunk_pages, float *part_o,
+                                  float *part_ml, const float *dist_r1, const float *dist_r2, int all_values,
+                                  const float *sink_scores, void *stream);
+
 // The same with the bias r1[h] ln(1 + r2[h] distance) taken off every score (dist_r1, dist_r2 f32 [heads_q], or both
 // NULL) and, with all_values, every query head's weights applied to the values of every kv head: out bf16
 // [rows, heads_q, heads_kv, dv], the scratch heads_kv times as large.
@@ -391,6 +400,20 @@ extern "C" int sb_cattn_shared_bf16(void *out, const void *q, const void *k_cach
                                     int window, float softcap, int sink, int chunks, int chunk_pages, float *part_o,
                                     float *part_ml, const float *dist_r1, const float *dist_r2, int all_values,
                                     void *stream) {
+  return sb_cattn_sink_bf16(out, q, k_cache, v_cache, page_table, max_pages, n_pages, row_pos, tiles, n_tiles, n_rows, heads_q,
+                            heads_kv, scale, window, softcap, sink, chunks, chunk_pages, part_o, part_ml, dist_r1, dist_r2,
+                            all_values, nullptr, stream);
+}
+
+// The same with a sink whose score is a number of the query head's own (sink_scores f32 [heads_q], as it is: not
+// scaled, not capped; NULL: 0).
+extern "C" int sb_cattn_sink_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
+                                  const int32_t *page_table, int max_pages, int n_pages, const int32_t *row_pos,
+                                  const int32_t *tiles, int n_tiles, int n_rows, int heads_q, int heads_kv, float scale,
+                                  int window, float softcap, int sink, int chunks, int chunk_pages, float *part_o,
+                                  float *part_ml, const float *dist_r1, const float *dist_r2, int all_values,
+                                  const float *sink_scores, void *stream) {
+  SB_REQUIRE(!sink_scores || sink, "sb_cattn_bf16: scores of a sink that is switched off");
   SB_REQUIRE((dist_r1 == nullptr) == (dist_r2 == nullptr), "sb_cattn_bf16: the distance bias needs both of its numbers");
   SB_REQUIRE(out && q && k_cache && v_cache && page_table && row_pos && tiles, "sb_cattn_bf16: null pointer");
   SB_REQUIRE(n_tiles >= 0 && n_rows >= 0 && heads_q > 0 && heads_kv > 0 && max_pages > 0 && n_pages > 0 && window >= 0,
@@ -415,6 +438,7 @@ extern "C" int sb_cattn_shared_bf16(void *out, const void *q, const void *k_cach
   a.window = window; a.sink = sink; a.chunk_pages = chunks == 1 ? 0 : chunk_pages;
   a.round_blocks = unsigned(sb::cu_count());
   a.dist_r1 = dist_r1; a.dist_r2 = dist_r2; a.all_values = all_values ? 1 : 0;
+  a.sink_scores = sink_scores;
   capped_attention_kernel<<<dim3(n_tiles, heads_kv * zgroups * value_heads, chunks), kThreads, 0, s>>>(a);
   int st = sb::check_launch("sb_cattn_bf16");
   if (st != SB_OK || chunks == 1) return st;

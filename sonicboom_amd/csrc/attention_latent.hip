@@ -39,7 +39,9 @@ latent_prepare_kernel(TA *__restrict__ q_plain, TA *__restrict__ q_latent, const
                       const float *__restrict__ inv_freq, int rot_dims, int interleaved,
                       const int32_t *__restrict__ row_pos, const int32_t *__restrict__ row_seq, TC *__restrict__ cache,
                       const int32_t *__restrict__ page_table, int max_pages, int n_pages_total, int heads, int dim,
-                      int rot_dim, int rank) {
+                      int rot_dim, int rank, const float *__restrict__ kv_rows, int kv_stride, float magnitude) {
+  // kv_rows (or NULL: p): the rows that hold the latent's part at kv_off, when the queries come from a
+  // product of their own; magnitude: multiplies every cosine and sine
   __shared__ double wave_part[kPrepThreads / 64];
   const int row = blockIdx.x, tid = threadIdx.x;
   const int pos = row_pos[row];
@@ -48,7 +50,7 @@ latent_prepare_kernel(TA *__restrict__ q_plain, TA *__restrict__ q_latent, const
   const float fpos = float(pos);
 
   if (kv_off >= 0) {                                  // this layer keeps its own latent: norm, rotate, store
-    const float *kv = pr + kv_off;
+    const float *kv = (kv_rows ? kv_rows + size_t(row) * kv_stride : pr) + kv_off;
     double part = 0.0;
     for (int i = tid; i < rank; i += kPrepThreads) part += double(kv[i] * kv[i]);
     part = wave_sum(part);
@@ -74,7 +76,8 @@ latent_prepare_kernel(TA *__restrict__ q_plain, TA *__restrict__ q_latent, const
         pair_index(j, rot_dims, interleaved, i0, i1);
         const float a = fpos * inv_freq[j];
         float y0, y1;
-        rotate_pair(r[i0], r[i1], cosf(a), sinf(a), y0, y1);
+        rotate_pair(r[i0], r[i1], magnitude == 1.0f ? cosf(a) : cosf(a) * magnitude,
+                    magnitude == 1.0f ? sinf(a) : sinf(a) * magnitude, y0, y1);
         st_f(dst, rank + i0, y0);
         st_f(dst, rank + i1, y1);
       }
@@ -97,7 +100,8 @@ latent_prepare_kernel(TA *__restrict__ q_plain, TA *__restrict__ q_latent, const
     const float *qr = q + a * hd + dim;
     const float ang = fpos * inv_freq[j];
     float y0, y1;
-    rotate_pair(qr[i0], qr[i1], cosf(ang), sinf(ang), y0, y1);
+    rotate_pair(qr[i0], qr[i1], magnitude == 1.0f ? cosf(ang) : cosf(ang) * magnitude,
+                magnitude == 1.0f ? sinf(ang) : sinf(ang) * magnitude, y0, y1);
     TA *dst = q_latent + (size_t(row) * heads + a) * latent + rank;
     st_f(dst, i0, y0);
     st_f(dst, i1, y1);
@@ -119,7 +123,7 @@ template <typename TO, typename TI, typename TW>
 __global__ void __launch_bounds__(kHeadThreads)
 head_product_kernel(TO *__restrict__ out, int out_stride, int out_hstride, const TI *__restrict__ in, int in_stride,
                     int in_hstride, const TW *__restrict__ w, const float *__restrict__ gate, int gate_stride,
-                    int n_rows, int n_in, int n_out) {
+                    int n_rows, int n_in, int n_out, int gate_per_head) {
   extern __shared__ float xin[];                    // [kHeadRows][n_in]
   const int a = blockIdx.y;
   const int t0 = blockIdx.x * kHeadRows;
@@ -145,7 +149,7 @@ head_product_kernel(TO *__restrict__ out, int out_stride, int out_hstride, const
       if (r >= nt) break;
       float v = acc[r];
       if (gate) {
-        const float g = gate[size_t(t0 + r) * gate_stride + size_t(a) * n_out + o];
+        const float g = gate[size_t(t0 + r) * gate_stride + (gate_per_head ? size_t(a) : size_t(a) * n_out + o)];
         v = v * (1.0f / (1.0f + expf(-g)));
       }
       st_f(out, size_t(t0 + r) * out_stride + size_t(a) * out_hstride + o, v);
@@ -231,19 +235,38 @@ latent_attention_kernel(TA *__restrict__ out, const TA *__restrict__ q, const TC
 //     [c | r] of the row's position in cache [pages, SB_PAGE, rank + rot_dim].
 // The first rot_dims of the rot_dim numbers turn, pair j by the angle float(pos) * inv_freq[j];
 // pairs are (2j, 2j + 1) when interleaved, else (j, j + rot_dims / 2).
+extern "C" int sb_latent_prepare_split(void *q_plain, void *q_latent, int act_dtype, const float *p, int row_stride,
+                                       int q_off, const float *kv_rows, int kv_stride, int kv_off, const void *c_weight,
+                                       int c_w_dtype, float eps, const float *inv_freq, int rot_dims, int interleaved,
+                                       float magnitude, const int32_t *row_pos, const int32_t *row_seq, void *cache,
+                                       int cache_dtype, const int32_t *page_table, int max_pages, int n_pages_total,
+                                       int n_rows, int heads, int dim, int rot_dim, int rank, void *stream);
 extern "C" int sb_latent_prepare(void *q_plain, void *q_latent, int act_dtype, const float *p, int row_stride,
                                  int q_off, int kv_off, const void *c_weight, int c_w_dtype, float eps,
                                  const float *inv_freq, int rot_dims, int interleaved, const int32_t *row_pos,
                                  const int32_t *row_seq, void *cache, int cache_dtype, const int32_t *page_table,
                                  int max_pages, int n_pages_total, int n_rows, int heads, int dim, int rot_dim,
                                  int rank, void *stream) {
+  return sb_latent_prepare_split(q_plain, q_latent, act_dtype, p, row_stride, q_off, nullptr, 0, kv_off, c_weight, c_w_dtype,
+                                 eps, inv_freq, rot_dims, interleaved, 1.0f, row_pos, row_seq, cache, cache_dtype, page_table,
+                                 max_pages, n_pages_total, n_rows, heads, dim, rot_dim, rank, stream);
+}
+
+// The same with the latent's part read at kv_off of rows of their own, kv_rows f32 [n_rows, kv_stride] (NULL: of p,
+// as above), for mixers whose queries come out of a second product, and with every cosine and sine times `magnitude`.
+extern "C" int sb_latent_prepare_split(void *q_plain, void *q_latent, int act_dtype, const float *p, int row_stride,
+                                       int q_off, const float *kv_rows, int kv_stride, int kv_off, const void *c_weight,
+                                       int c_w_dtype, float eps, const float *inv_freq, int rot_dims, int interleaved,
+                                       float magnitude, const int32_t *row_pos, const int32_t *row_seq, void *cache,
+                                       int cache_dtype, const int32_t *page_table, int max_pages, int n_pages_total,
+                                       int n_rows, int heads, int dim, int rot_dim, int rank, void *stream) {
   SB_REQUIRE(q_plain && q_latent && p && row_pos && row_seq, "sb_latent_prepare: null pointer");
   SB_REQUIRE(n_rows >= 0 && heads > 0 && dim > 0 && rot_dim >= 0 && rank > 0, "sb_latent_prepare: bad sizes");
   SB_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= rot_dim, "sb_latent_prepare: %d of %d numbers rotate",
              rot_dims, rot_dim);
   SB_REQUIRE(rot_dims == 0 || inv_freq, "sb_latent_prepare: a rotation needs its table");
   SB_REQUIRE(q_off >= 0 && q_off + heads * (dim + rot_dim) <= row_stride &&
-                 (kv_off < 0 || kv_off + rank + rot_dim <= row_stride),
+                 (kv_off < 0 || kv_off + rank + rot_dim <= (kv_rows ? kv_stride : row_stride)),
              "sb_latent_prepare: the parts do not fit a row of %d", row_stride);
   SB_REQUIRE(kv_off < 0 || (cache && page_table && max_pages > 0 && n_pages_total > 0),
              "sb_latent_prepare: a layer that stores needs its cache and page table");
@@ -255,7 +278,8 @@ extern "C" int sb_latent_prepare(void *q_plain, void *q_latent, int act_dtype, c
 #define SB_GO(TA, TC)                                                                                         \
   latent_prepare_kernel<TA, TC><<<n_rows, kPrepThreads, 0, s>>>(                                              \
       (TA *)q_plain, (TA *)q_latent, p, row_stride, q_off, kv_off, c_weight, c_w_dtype, eps, inv_freq, rot_dims, \
-      interleaved, row_pos, row_seq, (TC *)cache, page_table, max_pages, n_pages_total, heads, dim, rot_dim, rank)
+      interleaved, row_pos, row_seq, (TC *)cache, page_table, max_pages, n_pages_total, heads, dim, rot_dim, rank, \
+      kv_rows, kv_stride, magnitude)
   const int cdt = kv_off < 0 ? act_dtype : cache_dtype;
   if (act_dtype == SB_F32 && cdt == SB_F32) SB_GO(float, float);
   else if (act_dtype == SB_BF16 && cdt == SB_BF16) SB_GO(bf16_t, bf16_t);
@@ -269,10 +293,24 @@ extern "C" int sb_latent_prepare(void *q_plain, void *q_latent, int act_dtype, c
 // element (t, a, .) of out lies at t * out_stride + a * out_hstride, of in at t * in_stride +
 // a * in_hstride.  gate (f32, or NULL): the result is multiplied by sigmoid(gate[t * gate_stride +
 // a * n_out + o]).  in and W of one type (f32 or bf16), out f32 or bf16.
+extern "C" int sb_head_product_gated(void *out, int out_dtype, int out_stride, int out_hstride, const void *in,
+                                     int in_dtype, int in_stride, int in_hstride, const void *w, int w_dtype,
+                                     const float *gate, int gate_stride, int gate_per_head, int n_rows, int heads,
+                                     int n_in, int n_out, void *stream);
 extern "C" int sb_head_product(void *out, int out_dtype, int out_stride, int out_hstride, const void *in,
                                int in_dtype, int in_stride, int in_hstride, const void *w, int w_dtype,
                                const float *gate, int gate_stride, int n_rows, int heads, int n_in, int n_out,
                                void *stream) {
+  return sb_head_product_gated(out, out_dtype, out_stride, out_hstride, in, in_dtype, in_stride, in_hstride, w, w_dtype, gate,
+                               gate_stride, 0, n_rows, heads, n_in, n_out, stream);
+}
+
+// The same with gate_per_head: the gate holds one number a head, gate[t * gate_stride + a], for all of the
+// head's outputs.
+extern "C" int sb_head_product_gated(void *out, int out_dtype, int out_stride, int out_hstride, const void *in,
+                                     int in_dtype, int in_stride, int in_hstride, const void *w, int w_dtype,
+                                     const float *gate, int gate_stride, int gate_per_head, int n_rows, int heads,
+                                     int n_in, int n_out, void *stream) {
   SB_REQUIRE(out && in && w, "sb_head_product: null pointer");
   SB_REQUIRE(n_rows >= 0 && heads > 0 && n_in > 0 && n_out > 0, "sb_head_product: bad sizes");
   SB_REQUIRE(sb::valid_dtype(out_dtype) && sb::valid_dtype(in_dtype) && sb::valid_dtype(w_dtype),
@@ -286,7 +324,7 @@ extern "C" int sb_head_product(void *out, int out_dtype, int out_stride, int out
 #define SB_GO(TO, TI, TW)                                                                                      \
   head_product_kernel<TO, TI, TW><<<grid, kHeadThreads, lds, s>>>((TO *)out, out_stride, out_hstride, (const TI *)in, \
                                                                   in_stride, in_hstride, (const TW *)w, gate,         \
-                                                                  gate_stride, n_rows, n_in, n_out)
+                                                                  gate_stride, n_rows, n_in, n_out, gate_per_head)
   const int key = out_dtype * 4 + in_dtype * 2 + w_dtype;
   switch (key) {
     case 0: SB_GO(float, float, float); break;

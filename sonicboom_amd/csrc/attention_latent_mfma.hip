@@ -34,7 +34,7 @@ template <bool GATED>
 __global__ void __launch_bounds__(kThreads)
 head_product_mfma_kernel(bf16_t *__restrict__ out, int out_stride, int out_hstride, const bf16_t *__restrict__ in,
                          int in_stride, int in_hstride, const bf16_t *__restrict__ w, const float *__restrict__ gate,
-                         int gate_stride, int n_rows, int n_in, int n_out) {
+                         int gate_stride, int n_rows, int n_in, int n_out, int gate_per_head) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int a = blockIdx.y;
   const int t = blockIdx.x * 64 + wave * 16 + (lane & 15);      // this lane's row (B operand's column)
@@ -75,7 +75,7 @@ head_product_mfma_kernel(bf16_t *__restrict__ out, int out_stride, int out_hstri
     for (int i = 0; i < 4; ++i) {
       v[i] = acc[j][i];
       if (GATED && ob + i < n_out) {
-        const float gv = gate[size_t(t) * gate_stride + size_t(a) * n_out + ob + i];
+        const float gv = gate[size_t(t) * gate_stride + (gate_per_head ? size_t(a) : size_t(a) * n_out + ob + i)];
         v[i] = v[i] * (1.0f / (1.0f + expf(-gv)));
       }
     }
@@ -425,9 +425,21 @@ extern "C" int sb_head_product_bf16_ok(int out_stride, int out_hstride, int in_s
 
 // out[t, a, o] = sum_i W[a][o][i] in[t, a, i] on the matrix cores; everything bfloat16, gate f32 or NULL
 // (times sigmoid(gate[t * gate_stride + a * n_out + o])); in and W 16-byte aligned.
+extern "C" int sb_head_product_gated_bf16(void *out, int out_stride, int out_hstride, const void *in, int in_stride,
+                                          int in_hstride, const void *w, const float *gate, int gate_stride,
+                                          int gate_per_head, int n_rows, int heads, int n_in, int n_out, void *stream);
 extern "C" int sb_head_product_bf16(void *out, int out_stride, int out_hstride, const void *in, int in_stride,
                                     int in_hstride, const void *w, const float *gate, int gate_stride, int n_rows,
                                     int heads, int n_in, int n_out, void *stream) {
+  return sb_head_product_gated_bf16(out, out_stride, out_hstride, in, in_stride, in_hstride, w, gate, gate_stride, 0, n_rows,
+                                    heads, n_in, n_out, stream);
+}
+
+// The same with gate_per_head: the gate holds one number a head, gate[t * gate_stride + a], for all of the
+// head's outputs.
+extern "C" int sb_head_product_gated_bf16(void *out, int out_stride, int out_hstride, const void *in, int in_stride,
+                                          int in_hstride, const void *w, const float *gate, int gate_stride,
+                                          int gate_per_head, int n_rows, int heads, int n_in, int n_out, void *stream) {
   SB_REQUIRE(out && in && w, "sb_head_product_bf16: null pointer");
   SB_REQUIRE(n_rows >= 0 && heads > 0 && n_in > 0 && n_out > 0, "sb_head_product_bf16: bad sizes");
   SB_SUPPORT(sb_head_product_bf16_ok(out_stride, out_hstride, in_stride, in_hstride, n_in),
@@ -441,11 +453,11 @@ extern "C" int sb_head_product_bf16(void *out, int out_stride, int out_hstride, 
   if (gate)
     head_product_mfma_kernel<true><<<grid, kThreads, 0, s>>>((bf16_t *)out, out_stride, out_hstride, (const bf16_t *)in,
                                                              in_stride, in_hstride, (const bf16_t *)w, gate, gate_stride,
-                                                             n_rows, n_in, n_out);
+                                                             n_rows, n_in, n_out, gate_per_head);
   else
     head_product_mfma_kernel<false><<<grid, kThreads, 0, s>>>((bf16_t *)out, out_stride, out_hstride, (const bf16_t *)in,
                                                               in_stride, in_hstride, (const bf16_t *)w, gate, gate_stride,
-                                                              n_rows, n_in, n_out);
+                                                              n_rows, n_in, n_out, gate_per_head);
   return sb::check_launch("sb_head_product_bf16");
 }
 

@@ -29,7 +29,7 @@ attention_plain_kernel(TA *__restrict__ out, const TA *__restrict__ q, int q_str
                        const int32_t *__restrict__ page_table, int max_pages, int n_pages_total,
                        const int32_t *__restrict__ row_pos, const int32_t *__restrict__ row_seq,
                        int heads_q, int heads_kv, int head_dim, float scale, int window, int v_dim,
-                       float softcap, int sink) {
+                       float softcap, int sink, const float *__restrict__ sink_scores) {
   __shared__ float qs[kMaxHeadDim];
   __shared__ float ps[64];
   const int row = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -40,9 +40,10 @@ attention_plain_kernel(TA *__restrict__ out, const TA *__restrict__ q, int q_str
 
   const int lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
   const float neg_inf = -__builtin_inff();
-  // a sink is one more key of score 0 that has no value: the running maximum starts at its score
-  // and the running sum at its weight
-  float m = sink ? 0.0f : neg_inf, l = sink ? 1.0f : 0.0f;
+  // a sink is one more key that has no value, of score 0 or, with sink_scores, of the head's own
+  // number (as it is: no scale, no cap): the running maximum starts at its score and the running
+  // sum at its weight
+  float m = sink ? (sink_scores ? sink_scores[h] : 0.0f) : neg_inf, l = sink ? 1.0f : 0.0f;
   float o[kMaxHeadDim / 64] = {0.0f, 0.0f, 0.0f, 0.0f};
 
   for (int c = lo / SB_PAGE; c <= pos / SB_PAGE; ++c) {
@@ -110,12 +111,33 @@ extern "C" int sb_attention(void *out, const void *q, int act_dtype, int q_strid
                              window, 0.0f, 0, stream);
 }
 
+extern "C" int sb_attention_sink(void *out, const void *q, int act_dtype, int q_stride, const void *k_cache,
+                                 const void *v_cache, int cache_dtype, const int32_t *page_table,
+                                 int max_pages, int n_pages_total, const int32_t *row_pos,
+                                 const int32_t *row_seq, int n_rows, int heads_q, int heads_kv,
+                                 int head_dim, int v_dim, float scale, int window, float softcap, int sink,
+                                 const float *sink_scores, void *stream);
+
 extern "C" int sb_attention_capped(void *out, const void *q, int act_dtype, int q_stride, const void *k_cache,
                                    const void *v_cache, int cache_dtype, const int32_t *page_table,
                                    int max_pages, int n_pages_total, const int32_t *row_pos,
                                    const int32_t *row_seq, int n_rows, int heads_q, int heads_kv,
                                    int head_dim, int v_dim, float scale, int window, float softcap, int sink,
                                    void *stream) {
+  return sb_attention_sink(out, q, act_dtype, q_stride, k_cache, v_cache, cache_dtype, page_table, max_pages, n_pages_total,
+                           row_pos, row_seq, n_rows, heads_q, heads_kv, head_dim, v_dim, scale, window, softcap, sink,
+                           nullptr, stream);
+}
+
+// The same with a sink whose score is a number of the query head's own, sink_scores f32 [heads_q]
+// (NULL: 0): weights exp(s_j) / (exp(sink_h) + sum exp(s_j)).
+extern "C" int sb_attention_sink(void *out, const void *q, int act_dtype, int q_stride, const void *k_cache,
+                                 const void *v_cache, int cache_dtype, const int32_t *page_table,
+                                 int max_pages, int n_pages_total, const int32_t *row_pos,
+                                 const int32_t *row_seq, int n_rows, int heads_q, int heads_kv,
+                                 int head_dim, int v_dim, float scale, int window, float softcap, int sink,
+                                 const float *sink_scores, void *stream) {
+  SB_REQUIRE(!sink_scores || sink, "sb_attention: scores of a sink that is switched off");
   SB_REQUIRE(out && q && k_cache && v_cache && page_table && row_pos && row_seq,
              "sb_attention: null pointer");
   SB_REQUIRE(n_rows >= 0 && heads_q > 0 && heads_kv > 0 && head_dim > 0 && max_pages > 0 &&
@@ -138,7 +160,7 @@ extern "C" int sb_attention_capped(void *out, const void *q, int act_dtype, int 
   attention_plain_kernel<TA, TC><<<grid, 64, 0, s>>>(                                            \
       (TA *)out, (const TA *)q, q_stride, (const TC *)k_cache, (const TC *)v_cache, page_table,  \
       max_pages, n_pages_total, row_pos, row_seq, heads_q, heads_kv, head_dim, scale, window, v_dim,  \
-      softcap, sink)
+      softcap, sink, sink_scores)
   if (act_dtype == SB_F32 && cache_dtype == SB_F32) SB_GO(float, float);
   else if (act_dtype == SB_BF16 && cache_dtype == SB_BF16) SB_GO(bf16_t, bf16_t);
   else if (act_dtype == SB_F32 && cache_dtype == SB_BF16) SB_GO(float, bf16_t);

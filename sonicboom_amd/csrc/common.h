@@ -54,6 +54,14 @@ __device__ __forceinline__ float expert_pair(float g, float u, int kind, float l
   return swish_clamp_mul(g, u, limit, alpha);
 }
 
+// Values of the experts' products' `gated` argument that are no pair: 0 the product as it is, 3 an expert
+// without a gate whose activation is the square of max(z, 0).  1 and 2 are pairs (two matrix rows an output).
+__device__ __host__ __forceinline__ bool expert_is_pair(int kind) { return kind == 1 || kind == 2; }
+__device__ __forceinline__ float expert_single(float z, int kind) {
+  if (kind == 3) { const float r = fmaxf(z, 0.0f); return r * r; }
+  return z;
+}
+
 // The rotation of one pair (x0, x1) by the angle whose cosine and sine are c and s: every product
 // and sum rounded on its own (no fused multiply-add), so that every kernel that rotates a pair
 // gives the same bits (/root/reference/core/src/nn/rope.cpp:46-55).

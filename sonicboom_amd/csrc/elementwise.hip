@@ -102,6 +102,8 @@ __device__ __forceinline__ float softplus_f(float a) { return a > 20.0f ? a : lo
 // (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2.
 __device__ __forceinline__ float activate_one(float z, int kind, float ap, float an) {
   if (kind == SB_ACT_XIELU) return z > 0.0f ? ap * z * z + 0.5f * z : an * (expm1f(z) - z) + 0.5f * z;
+  if (kind == SB_ACT_GELU_ERF) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752440f));      // z Phi(z) by the error function
+  if (kind == SB_ACT_RELU_SQ) { const float r = fmaxf(z, 0.0f); return r * r; }
   return gate_act(z, kind == SB_ACT_GELU_TANH ? SB_GATE_GELU_TANH : SB_GATE_SILU);
 }
 
@@ -156,7 +158,7 @@ extern "C" int sb_activate(void *out, int out_dtype, const void *in, int in_dtyp
                            const void *params, int params_dtype, void *stream) {
   SB_REQUIRE(out && in, "sb_activate: null pointer");
   SB_REQUIRE(sb::valid_dtype(out_dtype) && sb::valid_dtype(in_dtype), "sb_activate: unknown dtype");
-  SB_SUPPORT(kind == SB_ACT_SILU || kind == SB_ACT_GELU_TANH || kind == SB_ACT_XIELU,
+  SB_SUPPORT(kind == SB_ACT_SILU || kind == SB_ACT_GELU_TANH || kind == SB_ACT_XIELU || kind == SB_ACT_GELU_ERF || kind == SB_ACT_RELU_SQ,
              "sb_activate: unknown activation %d", kind);
   SB_REQUIRE(kind != SB_ACT_XIELU || (params && sb::valid_dtype(params_dtype)),
              "sb_activate: xIELU needs its two numbers");
@@ -173,6 +175,49 @@ extern "C" int sb_activate(void *out, int out_dtype, const void *in, int in_dtyp
   else SB_GO(float, bf16_t);
 #undef SB_GO
   return sb::check_launch("sb_activate");
+}
+
+// ---- a sigmoid gate on finished rows, and a cap on logits ------------------------------------------------
+namespace {
+
+// x[t, i] *= sigmoid(gate[t * gate_stride + i]): x in the activation type, the gate's rows float32
+// (a part of a wider product's rows).  The sigmoid in float32 with the full-precision exponential.
+template <typename TX>
+__global__ void sigmoid_mul_kernel(TX *__restrict__ x, const float *__restrict__ gate, int gate_stride, int width, size_t n) {
+  const size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const size_t t = idx / width, i = idx - t * width;
+  const float g = gate[t * gate_stride + i];
+  st_f(x, idx, ld_f(x, idx) * (1.0f / (1.0f + expf(-g))));
+}
+
+__global__ void softcap_kernel(float *__restrict__ x, float cap, size_t n) {
+  const size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx < n) x[idx] = cap * tanhf(x[idx] / cap);
+}
+
+}  // namespace
+
+extern "C" int sb_sigmoid_mul(void *x, int x_dtype, const float *gate, int gate_stride, int n_rows, int width, void *stream) {
+  SB_REQUIRE(x && gate, "sb_sigmoid_mul: null pointer");
+  SB_REQUIRE(n_rows >= 0 && width > 0 && gate_stride >= width && sb::valid_dtype(x_dtype),
+             "sb_sigmoid_mul: bad sizes rows=%d width=%d stride=%d", n_rows, width, gate_stride);
+  const size_t n = size_t(n_rows) * width;
+  if (n == 0) return SB_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned nb = blocks_for(n, 256);
+  if (x_dtype == SB_F32) sigmoid_mul_kernel<float><<<nb, 256, 0, s>>>((float *)x, gate, gate_stride, width, n);
+  else sigmoid_mul_kernel<bf16_t><<<nb, 256, 0, s>>>((bf16_t *)x, gate, gate_stride, width, n);
+  return sb::check_launch("sb_sigmoid_mul");
+}
+
+// x <- cap tanh(x / cap), element by element, float32 in place (logits).
+extern "C" int sb_softcap(float *x, float cap, size_t n, void *stream) {
+  SB_REQUIRE(x, "sb_softcap: null pointer");
+  SB_REQUIRE(cap > 0.0f, "sb_softcap: the cap must be positive");
+  if (n == 0) return SB_OK;
+  softcap_kernel<<<blocks_for(n, 256), 256, 0, (hipStream_t)stream>>>(x, cap, n);
+  return sb::check_launch("sb_softcap");
 }
 
 // ---- measurement: how fast can this GPU stream memory? ---------------------------------------

@@ -93,11 +93,15 @@ __device__ __forceinline__ void write_normed(TO *yr, const float4 &v, int g, flo
 template <typename TO, int kNormThreads, int kNormKeep>
 __global__ void __launch_bounds__(kNormThreads)
 rmsnorm_kernel(TO *__restrict__ y, const float *__restrict__ x, const void *__restrict__ w,
-               int w_dtype, const int32_t *__restrict__ rows, int width, float eps) {
+               int w_dtype, const int32_t *__restrict__ rows, int width, float eps, int x_stride = 0,
+               TO *__restrict__ y2 = nullptr, const void *__restrict__ w2 = nullptr) {
+  // x_stride: the distance between rows of x when they are parts of wider rows (0: the width).
+  // y2, w2: a second result of the same rows with a weight of its own (one root mean square for both).
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
-  const float *xr = x + size_t(src) * width;
+  const float *xr = x + size_t(src) * (x_stride ? x_stride : width);
   TO *yr = y + size_t(r) * width;
+  TO *yr2 = y2 ? y2 + size_t(r) * width : nullptr;
   const int tid = threadIdx.x;
   const bool vec = (width % 4 == 0) && (reinterpret_cast<uintptr_t>(xr) % 16 == 0);
   const int n_groups = vec ? width / 4 : 0;
@@ -123,12 +127,15 @@ rmsnorm_kernel(TO *__restrict__ y, const float *__restrict__ x, const void *__re
 #pragma unroll
   for (int i = 0; i < kNormKeep; ++i) {
     const int g = tid + i * kNormThreads;
-    if (g < n_groups) write_normed(yr, keep[i], g, inv, w, w_dtype);
+    if (g < n_groups) {
+      write_normed(yr, keep[i], g, inv, w, w_dtype);
+      if (yr2) write_normed(yr2, keep[i], g, inv, w2, w_dtype);
+    }
   }
   for (int i = tail0 + tid; i < width; i += kNormThreads) {
-    float o = xr[i] * inv;
-    if (w) o = o * ld_dyn(w, w_dtype, i);
-    st_f(yr, i, o);
+    const float n = xr[i] * inv;
+    st_f(yr, i, w ? n * ld_dyn(w, w_dtype, i) : n);
+    if (yr2) st_f(yr2, i, w2 ? n * ld_dyn(w2, w_dtype, i) : n);
   }
 }
 
@@ -428,4 +435,28 @@ extern "C" int sb_rmsnorm(void *y, int out_dtype, const float *x, const void *w,
     else rmsnorm_kernel<bf16_t, 1024, 2><<<n_rows, 1024, 0, s>>>((bf16_t *)y, x, w, w_dtype, rows, width, eps);
   }
   return sb::check_launch("sb_rmsnorm");
+}
+
+// Two RMS norms of the same rows in one pass: y1 = (x inv) w1 and, when y2 is given, y2 = (x inv) w2,
+// with one root mean square for both (two branches that read the same stream through norms of
+// their own).  x_stride: the distance between rows of x (at least width), so that a part of wider
+// rows can be normed where it lies.  The arithmetic of every number is sb_rmsnorm's.
+extern "C" int sb_rmsnorm_pair(void *y1, void *y2, int out_dtype, const float *x, int x_stride, const void *w1,
+                               const void *w2, int w_dtype, int n_rows, int width, float eps, void *stream) {
+  SB_REQUIRE(y1 && x, "sb_rmsnorm_pair: null pointer");
+  SB_REQUIRE(n_rows >= 0 && width > 0 && x_stride >= width, "sb_rmsnorm_pair: bad sizes rows=%d width=%d stride=%d", n_rows,
+             width, x_stride);
+  SB_REQUIRE(sb::valid_dtype(out_dtype) && ((!w1 && !w2) || sb::valid_dtype(w_dtype)), "sb_rmsnorm_pair: unknown dtype");
+  SB_REQUIRE(eps >= 0.0f, "sb_rmsnorm_pair: eps must not be negative");
+  if (n_rows == 0) return SB_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const bool many = n_rows >= 256;
+  if (out_dtype == SB_F32) {
+    rmsnorm_kernel<float, 1024, 2><<<n_rows, 1024, 0, s>>>((float *)y1, x, w1, w_dtype, nullptr, width, eps, x_stride, (float *)y2, w2);
+  } else {
+    if (many && width > 4096) rmsnorm_kernel<bf16_t, 256, 8><<<n_rows, 256, 0, s>>>((bf16_t *)y1, x, w1, w_dtype, nullptr, width, eps, x_stride, (bf16_t *)y2, w2);
+    else if (many) rmsnorm_kernel<bf16_t, 256, 4><<<n_rows, 256, 0, s>>>((bf16_t *)y1, x, w1, w_dtype, nullptr, width, eps, x_stride, (bf16_t *)y2, w2);
+    else rmsnorm_kernel<bf16_t, 1024, 2><<<n_rows, 1024, 0, s>>>((bf16_t *)y1, x, w1, w_dtype, nullptr, width, eps, x_stride, (bf16_t *)y2, w2);
+  }
+  return sb::check_launch("sb_rmsnorm_pair");
 }

@@ -22,14 +22,37 @@ constexpr int kMaxTop = 16;
 // number), the softmax over them, the gate.
 // score_kind 0: the weights are the softmax over the chosen z.  score_kind 1: the scores are sigmoid(z), the
 // largest scores are chosen and the weights are those scores times score_scale, not renormalized.
+// score_kind 2: the scores are the softmax of z over all experts; the largest are chosen (the order of z) and the
+// weights are those scores times score_scale, not renormalized.
+// n_groups > 1: the experts lie in that many equal groups of neighbours, a group's score is its largest score, and
+// only experts of the keep_groups best groups (ties to the lower number) can be chosen.
 __device__ __forceinline__ void route_row(int32_t *__restrict__ ids, float *__restrict__ weights, const float *zr, int r,
-                                          int n_experts, int top, int has_gate, int score_kind = 0, float score_scale = 1.0f) {
+                                          int n_experts, int top, int has_gate, int score_kind = 0, float score_scale = 1.0f,
+                                          int n_groups = 1, int keep_groups = 1) {
   int chosen[kMaxTop];
   float score[kMaxTop];
+  unsigned long long open_groups = ~0ull;       // bit g: experts of group g can be chosen
+  const int per_group = n_groups > 1 ? n_experts / n_groups : n_experts;
+  if (n_groups > 1 && keep_groups < n_groups) {
+    // (every kind of score rises with z, so the groups are ranked by their largest z)
+    open_groups = 0ull;
+    for (int k = 0; k < keep_groups; ++k) {
+      int best = -1;
+      float bz = 0.0f;
+      for (int g = 0; g < n_groups; ++g) {
+        if ((open_groups >> g) & 1ull) continue;
+        float gz = -__builtin_inff();
+        for (int e = g * per_group; e < (g + 1) * per_group; ++e) gz = fmaxf(gz, zr[e]);
+        if (best < 0 || gz > bz) { best = g; bz = gz; }
+      }
+      open_groups |= 1ull << best;
+    }
+  }
   for (int k = 0; k < top; ++k) {
     int best = -1;
     float bz = 0.0f;
     for (int e = 0; e < n_experts; ++e) {
+      if (n_groups > 1 && !((open_groups >> (e / per_group)) & 1ull)) continue;
       const float v = score_kind == 1 ? 1.0f / (1.0f + expf(-zr[e])) : zr[e];
       // candidates: below the last choice, or equal to it with a higher number (the order is
       // falling scores, rising numbers among equals); NaN scores are never chosen
@@ -41,20 +64,29 @@ __device__ __forceinline__ void route_row(int32_t *__restrict__ ids, float *__re
     score[k] = bz;
   }
   float sum = 0.0f, w[kMaxTop];
-  for (int k = 0; k < top; ++k) { w[k] = expf(score[k] - score[0]); sum += w[k]; }
+  if (score_kind == 2) {
+    // the softmax over all experts: the largest z of all, then the sum in ascending order of the experts
+    float top_z = -__builtin_inff();
+    for (int e = 0; e < n_experts; ++e) top_z = fmaxf(top_z, zr[e]);
+    for (int e = 0; e < n_experts; ++e) sum += expf(zr[e] - top_z);
+    for (int k = 0; k < top; ++k) w[k] = expf(score[k] - top_z);
+  } else {
+    for (int k = 0; k < top; ++k) { w[k] = expf(score[k] - score[0]); sum += w[k]; }
+  }
   for (int k = 0; k < top; ++k) {
     ids[size_t(r) * top + k] = chosen[k];
-    weights[size_t(r) * (top + 1) + k] = score_kind == 1 ? score[k] * score_scale : w[k] / sum;
+    weights[size_t(r) * (top + 1) + k] = score_kind == 1 ? score[k] * score_scale : score_kind == 2 ? (w[k] / sum) * score_scale : w[k] / sum;
   }
   weights[size_t(r) * (top + 1) + top] = has_gate ? 1.0f / (1.0f + expf(-zr[n_experts])) : 0.0f;
 }
 
 __global__ void __launch_bounds__(64)
 moe_route_kernel(int32_t *__restrict__ ids, float *__restrict__ weights, const float *__restrict__ z, int n_rows,
-                 int stride, int n_experts, int top, int has_gate, int score_kind, float score_scale) {
+                 int stride, int n_experts, int top, int has_gate, int score_kind, float score_scale, int n_groups,
+                 int keep_groups) {
   const int r = blockIdx.x * 64 + threadIdx.x;
   if (r >= n_rows) return;
-  route_row(ids, weights, z + size_t(r) * stride, r, n_experts, top, has_gate, score_kind, score_scale);
+  route_row(ids, weights, z + size_t(r) * stride, r, n_experts, top, has_gate, score_kind, score_scale, n_groups, keep_groups);
 }
 
 // The router's product and the choice in one launch: a block a row.  z_e = sum_k h[k] w[e][k] in
@@ -78,7 +110,7 @@ template <typename TX>
 __global__ void __launch_bounds__(256)
 moe_router_kernel(int32_t *__restrict__ ids, float *__restrict__ weights, const TX *__restrict__ h,
                   const float *__restrict__ w, int n_rows, int n_in, int n_experts, int top, int has_gate, int score_kind,
-                  float score_scale) {
+                  float score_scale, int n_groups, int keep_groups) {
   extern __shared__ float zs[];                 // [n_z] scores, then [4][8] the waves' sums of a pass
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int r = blockIdx.x;
@@ -119,7 +151,7 @@ moe_router_kernel(int32_t *__restrict__ ids, float *__restrict__ weights, const 
     if (tid < 8 && e0 + tid < n_z) z[e0 + tid] = ((part[tid] + part[8 + tid]) + part[16 + tid]) + part[24 + tid];
     __syncthreads();
   }
-  if (tid == 0) route_row(ids, weights, z, r, n_experts, top, has_gate, score_kind, score_scale);
+  if (tid == 0) route_row(ids, weights, z, r, n_experts, top, has_gate, score_kind, score_scale, n_groups, keep_groups);
 }
 
 template <typename TO>
@@ -145,11 +177,13 @@ moe_product_plain_kernel(TY *__restrict__ y, const TX *__restrict__ x, const TW 
   if (e < 0 || e >= n_experts) return;
   const int o = blockIdx.y * 256 + threadIdx.x;
   if (o >= n_out) return;
-  const size_t w_rows = size_t(gated ? 2 : 1) * n_out;
+  const bool pair = expert_is_pair(gated);
+  const size_t w_rows = size_t(pair ? 2 : 1) * n_out;
   const TW *wg = w + (size_t(e) * w_rows + o) * n_in;
   float g = 0.0f;
   for (int k = 0; k < n_in; ++k) g = fmaf(xs[k], ld_f(wg, k), g);
-  if (gated) {
+  if (!pair) g = expert_single(g, gated);
+  if (pair) {
     const TW *wu = wg + size_t(n_out) * n_in;
     float u = 0.0f;
     for (int k = 0; k < n_in; ++k) u = fmaf(xs[k], ld_f(wu, k), u);
@@ -169,15 +203,36 @@ extern "C" int sb_moe_route(int32_t *ids, float *weights, const float *z, int n_
   return sb_moe_route_scored(ids, weights, z, n_rows, stride, n_experts, top, has_gate, 0, 1.0f, stream);
 }
 
+extern "C" int sb_moe_route_grouped(int32_t *ids, float *weights, const float *z, int n_rows, int stride, int n_experts,
+                                    int top, int has_gate, int score_kind, float score_scale, int n_groups, int keep_groups,
+                                    void *stream);
 extern "C" int sb_moe_route_scored(int32_t *ids, float *weights, const float *z, int n_rows, int stride, int n_experts,
                                    int top, int has_gate, int score_kind, float score_scale, void *stream) {
+  return sb_moe_route_grouped(ids, weights, z, n_rows, stride, n_experts, top, has_gate, score_kind, score_scale, 1, 1, stream);
+}
+
+namespace {
+// 0 when the groups fit the experts and the choice: equal groups, enough experts in the groups that stay
+int check_groups(int n_experts, int top, int n_groups, int keep_groups) {
+  return n_groups >= 1 && n_groups <= 64 && n_experts % n_groups == 0 && keep_groups >= 1 && keep_groups <= n_groups &&
+         (n_groups == 1 || keep_groups * (n_experts / n_groups) >= top) ? 0 : 1;
+}
+}  // namespace
+
+// The same with score_kind 2 (softmax over all experts, weights not renormalized) and with the experts in n_groups
+// equal groups of neighbours of which the keep_groups with the largest best score can be chosen from.
+extern "C" int sb_moe_route_grouped(int32_t *ids, float *weights, const float *z, int n_rows, int stride, int n_experts,
+                                    int top, int has_gate, int score_kind, float score_scale, int n_groups, int keep_groups,
+                                    void *stream) {
   SB_REQUIRE(ids && weights && z, "sb_moe_route: null pointer");
-  SB_REQUIRE(score_kind == 0 || score_kind == 1, "sb_moe_route: unknown kind of score %d", score_kind);
+  SB_REQUIRE(score_kind >= 0 && score_kind <= 2, "sb_moe_route: unknown kind of score %d", score_kind);
+  SB_REQUIRE(check_groups(n_experts, top, n_groups, keep_groups) == 0, "sb_moe_route: %d of %d groups do not fit %d experts and %d choices",
+             keep_groups, n_groups, n_experts, top);
   SB_REQUIRE(n_rows >= 0 && n_experts > 0 && top > 0 && top <= n_experts && stride >= n_experts + (has_gate ? 1 : 0),
              "sb_moe_route: bad sizes rows=%d experts=%d top=%d stride=%d", n_rows, n_experts, top, stride);
   SB_SUPPORT(top <= kMaxTop, "sb_moe_route: %d choices a row are more than %d", top, kMaxTop);
   if (n_rows == 0) return SB_OK;
-  moe_route_kernel<<<(n_rows + 63) / 64, 64, 0, (hipStream_t)stream>>>(ids, weights, z, n_rows, stride, n_experts, top, has_gate, score_kind, score_scale);
+  moe_route_kernel<<<(n_rows + 63) / 64, 64, 0, (hipStream_t)stream>>>(ids, weights, z, n_rows, stride, n_experts, top, has_gate, score_kind, score_scale, n_groups, keep_groups);
   return sb::check_launch("sb_moe_route");
 }
 
@@ -189,11 +244,23 @@ extern "C" int sb_moe_router(int32_t *ids, float *weights, const void *h, int h_
   return sb_moe_router_scored(ids, weights, h, h_dtype, w, n_rows, n_in, n_experts, top, has_gate, 0, 1.0f, stream);
 }
 
+extern "C" int sb_moe_router_grouped(int32_t *ids, float *weights, const void *h, int h_dtype, const float *w, int n_rows,
+                                     int n_in, int n_experts, int top, int has_gate, int score_kind, float score_scale,
+                                     int n_groups, int keep_groups, void *stream);
 extern "C" int sb_moe_router_scored(int32_t *ids, float *weights, const void *h, int h_dtype, const float *w, int n_rows,
                                     int n_in, int n_experts, int top, int has_gate, int score_kind, float score_scale,
                                     void *stream) {
+  return sb_moe_router_grouped(ids, weights, h, h_dtype, w, n_rows, n_in, n_experts, top, has_gate, score_kind, score_scale, 1, 1,
+                               stream);
+}
+
+extern "C" int sb_moe_router_grouped(int32_t *ids, float *weights, const void *h, int h_dtype, const float *w, int n_rows,
+                                     int n_in, int n_experts, int top, int has_gate, int score_kind, float score_scale,
+                                     int n_groups, int keep_groups, void *stream) {
   SB_REQUIRE(ids && weights && h && w, "sb_moe_router: null pointer");
-  SB_REQUIRE(score_kind == 0 || score_kind == 1, "sb_moe_router: unknown kind of score %d", score_kind);
+  SB_REQUIRE(score_kind >= 0 && score_kind <= 2, "sb_moe_router: unknown kind of score %d", score_kind);
+  SB_REQUIRE(check_groups(n_experts, top, n_groups, keep_groups) == 0, "sb_moe_router: %d of %d groups do not fit %d experts and %d choices",
+             keep_groups, n_groups, n_experts, top);
   SB_REQUIRE(n_rows >= 0 && n_in > 0 && n_experts > 0 && top > 0 && top <= n_experts && sb::valid_dtype(h_dtype),
              "sb_moe_router: bad sizes rows=%d in=%d experts=%d top=%d", n_rows, n_in, n_experts, top);
   SB_SUPPORT(top <= kMaxTop && n_experts < 2048, "sb_moe_router: %d choices of %d experts are more than %d of 2047", top,
@@ -202,8 +269,8 @@ extern "C" int sb_moe_router_scored(int32_t *ids, float *weights, const void *h,
   hipStream_t s = (hipStream_t)stream;
   const size_t lds = size_t(n_experts + 1 + 32) * sizeof(float);
   const unsigned blocks = n_rows;
-  if (h_dtype == SB_F32) moe_router_kernel<float><<<blocks, 256, lds, s>>>(ids, weights, (const float *)h, w, n_rows, n_in, n_experts, top, has_gate, score_kind, score_scale);
-  else moe_router_kernel<bf16_t><<<blocks, 256, lds, s>>>(ids, weights, (const bf16_t *)h, w, n_rows, n_in, n_experts, top, has_gate, score_kind, score_scale);
+  if (h_dtype == SB_F32) moe_router_kernel<float><<<blocks, 256, lds, s>>>(ids, weights, (const float *)h, w, n_rows, n_in, n_experts, top, has_gate, score_kind, score_scale, n_groups, keep_groups);
+  else moe_router_kernel<bf16_t><<<blocks, 256, lds, s>>>(ids, weights, (const bf16_t *)h, w, n_rows, n_in, n_experts, top, has_gate, score_kind, score_scale, n_groups, keep_groups);
   return sb::check_launch("sb_moe_router");
 }
 

@@ -56,8 +56,9 @@ struct Args {
   void *y; int y_f32;
   const bf16_t *x, *w;
   const int32_t *order, *tiles, *n_tiles;      // NULL: one expert, the pairs in their own order
-  int n_pairs, x_div, n_out, n_in, gated;
+  int n_pairs, x_div, n_out, n_in, gated;      // gated: the kind of pair, 0 when an output is one matrix row
   float limit, alpha;
+  int single;                                  // the activation of an output that is no pair (expert_single)
 };
 
 // LDS place (in 16-byte chunks) of chunk c of row r of a tile whose rows are 8 chunks long
@@ -176,7 +177,8 @@ __global__ void __launch_bounds__(kThreads) moe_product_kernel(Args a) {
       for (int f = 0; f < (a.gated ? 2 : 4); ++f) {
         const int n = a.gated ? n0 + 32 * wc + 16 * f + col : n0 + 64 * wc + 16 * f + col;
         if (n >= a.n_out) continue;
-        const float v = a.gated ? expert_pair(acc[i][f][e], acc[i][f + 2][e], a.gated, a.limit, a.alpha) : acc[i][f][e];
+        const float v = a.gated ? expert_pair(acc[i][f][e], acc[i][f + 2][e], a.gated, a.limit, a.alpha)
+                                : expert_single(acc[i][f][e], a.single);
         if (a.y_f32) ((float *)a.y)[size_t(p) * a.n_out + n] = v;
         else ((bf16_t *)a.y)[size_t(p) * a.n_out + n] = f32_to_bf16(v);
       }
@@ -214,9 +216,10 @@ extern "C" int sb_moe_product_bf16(void *y, int y_dtype, const void *x, const vo
   SB_REQUIRE(sb::valid_dtype(y_dtype), "sb_moe_product_bf16: unknown dtype");
   SB_SUPPORT(n_in % 8 == 0, "sb_moe_product_bf16: an inner size of %d is no multiple of 8", n_in);
   if (n_pairs == 0) return SB_OK;
+  const bool pair = expert_is_pair(gated);
   const Args a{y, y_dtype == SB_F32 ? 1 : 0, (const bf16_t *)x, (const bf16_t *)w, order, tiles, n_tiles, n_pairs, x_div, n_out, n_in,
-               gated, limit, alpha};
-  const int n_cols = gated ? BN / 2 : BN;
+               pair ? gated : 0, limit, alpha, pair ? 0 : gated};
+  const int n_cols = pair ? BN / 2 : BN;
   const unsigned gx = tiles ? unsigned(max_tiles) : unsigned((n_pairs + tile_rows - 1) / tile_rows);
   const dim3 grid(gx, (n_out + n_cols - 1) / n_cols);
   SB_SUPPORT(grid.y <= 65535, "sb_moe_product_bf16: too many columns for one grid");

@@ -44,7 +44,10 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
                int rot_dims, const int32_t *__restrict__ row_pos,
                const int32_t *__restrict__ row_seq, TC *__restrict__ k_cache,
                TC *__restrict__ v_cache, const int32_t *__restrict__ page_table, int max_pages,
-               int n_pages_total, int heads_q, int heads_kv, int head_dim, int heads_per_block) {
+               int n_pages_total, int heads_q, int heads_kv, int head_dim, int heads_per_block, int v_dim,
+               float magnitude) {
+  // v_dim: numbers of a value head (the keys' head_dim unless the mixer's values have a size of their own);
+  // magnitude: multiplies every cosine and sine (1 unless the rotation's scaling stretches the vectors)
   const int row = blockIdx.x;
   const int pos = row_pos[row];
   const TI *r = qkv + size_t(row) * row_stride;
@@ -87,6 +90,7 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
   }
   const size_t head_step = size_t(SB_PAGE) * head_dim;  // from one kv head to the next within a page
   const size_t page_base = size_t(page_of_row) * heads_kv * head_step;
+  const size_t v_step = size_t(SB_PAGE) * v_dim, v_base = size_t(page_of_row) * heads_kv * v_step;
   const int slot = pos % SB_PAGE;      // keys [slot][d], values [d][slot], in the cache's order of groups
 
   // The angle of pair i is the same for every head of the row: cosine and sine once per block,
@@ -97,8 +101,8 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
       const int i = j < half ? j : j - half;
       float theta = float(pos) * inv_freq[i];
       if (freq_factors) theta = theta / freq_factors[i];
-      if (j < half) cs[i] = cosf(theta);
-      else sn[i] = sinf(theta);
+      if (j < half) cs[i] = magnitude == 1.0f ? cosf(theta) : cosf(theta) * magnitude;
+      else sn[i] = magnitude == 1.0f ? sinf(theta) : sinf(theta) * magnitude;
     }
   }
   __syncthreads();
@@ -110,10 +114,11 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
       // a value head: every element is copied, transposed into the page
       if (!store) continue;
       const int kh = head - heads_q - heads_kv;
+      const size_t voff = size_t(heads_q + heads_kv) * head_dim + size_t(kh) * v_dim;      // value heads lie behind all keys
 #pragma unroll 1
-      for (int d = w; d < head_dim; d += per_head)
-        st_f(v_cache, page_base + kh * head_step + sb_value_index(d, slot),
-             qkv_at<SLICES>(r, hoff + d, n_slices, slice_stride, bias));
+      for (int d = w; d < v_dim; d += per_head)
+        st_f(v_cache, v_base + kh * v_step + sb_value_index(d, slot),
+             qkv_at<SLICES>(r, voff + d, n_slices, slice_stride, bias));
       continue;
     }
     const bool is_q = head < heads_q;
@@ -192,7 +197,7 @@ rope_kv_rows_kernel(bf16_t *__restrict__ q_out, const TI *__restrict__ qkv, int 
                     const int32_t *__restrict__ row_pos, const int32_t *__restrict__ row_seq,
                     bf16_t *__restrict__ k_cache, bf16_t *__restrict__ v_cache,
                     const int32_t *__restrict__ page_table, int max_pages, int n_pages_total, int heads_q,
-                    int heads_kv, int head_dim) {
+                    int heads_kv, int head_dim, int v_dim, float magnitude) {
   const int row = blockIdx.x;
   const int pos = row_pos[row];
   const TI *r = qkv + size_t(row) * row_stride;
@@ -216,8 +221,8 @@ rope_kv_rows_kernel(bf16_t *__restrict__ q_out, const TI *__restrict__ qkv, int 
     const int i = j < half ? j : j - half;
     float theta = float(pos) * inv_freq[i];
     if (freq_factors) theta = theta / freq_factors[i];
-    if (j < half) cs[i] = cosf(theta);
-    else sn[i] = sinf(theta);
+    if (j < half) cs[i] = magnitude == 1.0f ? cosf(theta) : cosf(theta) * magnitude;
+    else sn[i] = magnitude == 1.0f ? sinf(theta) : sinf(theta) * magnitude;
   }
   __syncthreads();
   auto pack = [](const float (&f)[8]) {
@@ -255,17 +260,25 @@ rope_kv_rows_kernel(bf16_t *__restrict__ q_out, const TI *__restrict__ qkv, int 
   }
   // values: eight elements a time, each to its own row of the transposed page
   if (!store) return;
-  const int groups = head_dim / 8;
+  const int groups = v_dim / 8;
+  const size_t v_step = size_t(SB_PAGE) * v_dim, v_base = size_t(page_of_row) * heads_kv * v_step;
   for (int it = threadIdx.x; it < heads_kv * groups; it += blockDim.x) {
     const int kh = it / groups, d0 = (it % groups) * 8;
     float v[8];
-    qkv_eight<SLICES>(v, r, size_t(heads_q + heads_kv + kh) * head_dim + d0, n_slices, slice_stride, bias);
+    qkv_eight<SLICES>(v, r, size_t(heads_q + heads_kv) * head_dim + size_t(kh) * v_dim + d0, n_slices, slice_stride, bias);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v_cache[page_base + kh * head_step + sb_value_index(d0 + e, slot)] = f32_to_bf16(v[e]);
+    for (int e = 0; e < 8; ++e) v_cache[v_base + kh * v_step + sb_value_index(d0 + e, slot)] = f32_to_bf16(v[e]);
   }
 }
 
 }  // namespace
+
+extern "C" int sb_rope_kv_store_sized(void *q_out, int q_dtype, const void *qkv, int qkv_dtype,
+                                      int row_stride, int n_slices, const float *bias, const float *inv_freq, const float *freq_factors,
+                                      int rot_dims, const int32_t *row_pos, const int32_t *row_seq,
+                                      void *k_cache, void *v_cache, int cache_dtype,
+                                      const int32_t *page_table, int max_pages, int n_pages_total,
+                                      int n_rows, int heads_q, int heads_kv, int head_dim, int v_dim, float magnitude, void *stream);
 
 extern "C" int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int qkv_dtype,
                                 int row_stride, int n_slices, const float *bias, const float *inv_freq, const float *freq_factors,
@@ -273,14 +286,28 @@ extern "C" int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int q
                                 void *k_cache, void *v_cache, int cache_dtype,
                                 const int32_t *page_table, int max_pages, int n_pages_total,
                                 int n_rows, int heads_q, int heads_kv, int head_dim, void *stream) {
+  return sb_rope_kv_store_sized(q_out, q_dtype, qkv, qkv_dtype, row_stride, n_slices, bias, inv_freq, freq_factors, rot_dims, row_pos,
+                                row_seq, k_cache, v_cache, cache_dtype, page_table, max_pages, n_pages_total, n_rows, heads_q,
+                                heads_kv, head_dim, head_dim, 1.0f, stream);
+}
+
+// The same for value heads of v_dim numbers (a qkv row is [heads_q x head_dim | heads_kv x head_dim | heads_kv x v_dim],
+// the value pages [page][kv head][v_dim][position]) and with every cosine and sine times `magnitude`.
+extern "C" int sb_rope_kv_store_sized(void *q_out, int q_dtype, const void *qkv, int qkv_dtype,
+                                      int row_stride, int n_slices, const float *bias, const float *inv_freq, const float *freq_factors,
+                                      int rot_dims, const int32_t *row_pos, const int32_t *row_seq,
+                                      void *k_cache, void *v_cache, int cache_dtype,
+                                      const int32_t *page_table, int max_pages, int n_pages_total,
+                                      int n_rows, int heads_q, int heads_kv, int head_dim, int v_dim, float magnitude, void *stream) {
   SB_REQUIRE(qkv && row_pos, "sb_rope_kv_store: null pointer");
+  SB_REQUIRE(v_dim > 0, "sb_rope_kv_store: the values' size must be positive");
   SB_REQUIRE(n_rows >= 0 && heads_q >= 0 && heads_kv >= 0 && head_dim > 0 && heads_q + heads_kv > 0,
              "sb_rope_kv_store: bad sizes rows=%d heads_q=%d heads_kv=%d head_dim=%d", n_rows, heads_q,
              heads_kv, head_dim);
   SB_REQUIRE(heads_q == 0 || q_out, "sb_rope_kv_store: no buffer for the rotated queries");
-  SB_REQUIRE(row_stride >= (heads_q + 2 * heads_kv) * head_dim,
+  SB_REQUIRE(row_stride >= (heads_q + heads_kv) * head_dim + heads_kv * v_dim,
              "sb_rope_kv_store: row stride %d is shorter than a qkv row of %d", row_stride,
-             (heads_q + 2 * heads_kv) * head_dim);
+             (heads_q + heads_kv) * head_dim + heads_kv * v_dim);
   SB_REQUIRE(sb::valid_dtype(q_dtype) && sb::valid_dtype(qkv_dtype) && sb::valid_dtype(cache_dtype),
              "sb_rope_kv_store: unknown dtype");
   SB_REQUIRE(n_slices >= 1, "sb_rope_kv_store: at least one slice");
@@ -301,13 +328,13 @@ extern "C" int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int q
   const uintptr_t addresses = reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(q_out) |
                               reinterpret_cast<uintptr_t>(k_cache);
   const uintptr_t bias_address = reinterpret_cast<uintptr_t>(bias);
-  if (n_rows >= 512 && q_dtype == SB_BF16 && cache_dtype == SB_BF16 && head_dim % 8 == 0 && row_stride % 8 == 0 &&
+  if (n_rows >= 512 && q_dtype == SB_BF16 && cache_dtype == SB_BF16 && head_dim % 8 == 0 && v_dim % 8 == 0 && row_stride % 8 == 0 &&
       (!inv_freq || rot_dims % 16 == 0) && (addresses | bias_address) % 16 == 0) {
 #define SB_ROWS(TI, SLICES)                                                                              \
   rope_kv_rows_kernel<TI, SLICES><<<n_rows, 256, 0, s>>>(                                                \
       (bf16_t *)q_out, (const TI *)qkv, row_stride, n_slices, slice_stride, bias, inv_freq, freq_factors, \
       rot_dims, row_pos, row_seq, (bf16_t *)k_cache, (bf16_t *)v_cache, page_table, max_pages,           \
-      n_pages_total, heads_q, heads_kv, head_dim)
+      n_pages_total, heads_q, heads_kv, head_dim, v_dim, magnitude)
     if (qkv_dtype == SB_BF16) {
       if (n_slices == 1) SB_ROWS(bf16_t, 1);
       else if (n_slices <= 4) SB_ROWS(bf16_t, 4);
@@ -332,7 +359,7 @@ extern "C" int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int q
       (TQ *)q_out, (const TI *)qkv, row_stride, n_slices, slice_stride, bias, inv_freq, freq_factors,   \
       rot_dims, row_pos, row_seq,                                                                    \
       (TC *)k_cache, (TC *)v_cache, page_table, max_pages, n_pages_total, heads_q, heads_kv, head_dim,  \
-      heads_per_block)
+      heads_per_block, v_dim, magnitude)
   const int key = qkv_dtype * 4 + q_dtype * 2 + cache_dtype;
   switch (key) {
     case 0: SB_GO(float, float, float); break;

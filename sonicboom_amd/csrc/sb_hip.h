@@ -76,7 +76,7 @@ typedef enum sb_gate { SB_GATE_NONE = 0, SB_GATE_SILU = 1, SB_GATE_GELU_TANH = 2
 
 /* The `kind` argument of sb_activate.  xIELU takes two numbers (p, q) from memory: for z > 0
  * softplus(p) z^2 + z/2, else (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2. */
-typedef enum sb_act { SB_ACT_SILU = 1, SB_ACT_GELU_TANH = 2, SB_ACT_XIELU = 3 } sb_act;
+typedef enum sb_act { SB_ACT_SILU = 1, SB_ACT_GELU_TANH = 2, SB_ACT_XIELU = 3, SB_ACT_GELU_ERF = 4, SB_ACT_RELU_SQ = 5 } sb_act;
 
 /* Message of this thread's last failed call ("" if none). Never NULL. */
 const char *sb_last_error(void);
@@ -479,6 +479,49 @@ int sb_gemm_mfma_partial_bf16(float *partial, const void *x, const void *w, int 
  * host computes the same bits (sonicboom_amd/weights/random_stream.py). */
 int sb_random_normal(void *out, int out_kind, uint64_t n, uint64_t first, uint64_t seed, int tensor_index,
                      double mean, double std, void *stream);
+
+/* ---- later forms of the kernels above: the shorter entry points call them with the arguments that
+ * make them what they were ------------------------------------------------------------------------
+ * sb_rmsnorm_pair: two RMS norms of the same rows (one root mean square, two weights, y2 may be NULL),
+ *   the rows x_stride apart (parts of wider rows).
+ * sb_sigmoid_mul: x[t, i] *= sigmoid(gate[t * gate_stride + i]).  sb_softcap: x <- cap tanh(x / cap).
+ * sb_rope_kv_store_sized: value heads of v_dim numbers; every cosine and sine times `magnitude`.
+ * sb_attention_sink: the sink's score a number of the query head's own (sink_scores f32 [heads_q]).
+ * sb_latent_prepare_split: the latent's part read from rows of its own; `magnitude` as above.
+ * sb_head_product_gated(_bf16): gate_per_head, one gate number a head.
+ * sb_moe_route_grouped / sb_moe_router_grouped: score_kind 0 softmax over the chosen, 1 sigmoid, 2 softmax
+ *   over all experts (weights not renormalized); experts in n_groups equal groups of neighbours of which
+ *   the keep_groups with the largest best score can be chosen from.
+ * The experts' products' `gated`: 0 as it is, 1 and 2 pairs, 3 one matrix row an output and max(z, 0)^2. */
+int sb_rmsnorm_pair(void *y1, void *y2, int out_dtype, const float *x, int x_stride, const void *w1, const void *w2,
+                    int w_dtype, int n_rows, int width, float eps, void *stream);
+int sb_sigmoid_mul(void *x, int x_dtype, const float *gate, int gate_stride, int n_rows, int width, void *stream);
+int sb_softcap(float *x, float cap, size_t n, void *stream);
+int sb_rope_kv_store_sized(void *q_out, int q_dtype, const void *qkv, int qkv_dtype, int row_stride, int n_slices,
+                           const float *bias, const float *inv_freq, const float *freq_factors, int rot_dims,
+                           const int32_t *row_pos, const int32_t *row_seq, void *k_cache, void *v_cache, int cache_dtype,
+                           const int32_t *page_table, int max_pages, int n_pages_total, int n_rows, int heads_q,
+                           int heads_kv, int head_dim, int v_dim, float magnitude, void *stream);
+int sb_attention_sink(void *out, const void *q, int act_dtype, int q_stride, const void *k_cache, const void *v_cache,
+                      int cache_dtype, const int32_t *page_table, int max_pages, int n_pages_total,
+                      const int32_t *row_pos, const int32_t *row_seq, int n_rows, int heads_q, int heads_kv, int head_dim,
+                      int v_dim, float scale, int window, float softcap, int sink, const float *sink_scores, void *stream);
+int sb_latent_prepare_split(void *q_plain, void *q_latent, int act_dtype, const float *p, int row_stride, int q_off,
+                            const float *kv_rows, int kv_stride, int kv_off, const void *c_weight, int c_w_dtype, float eps,
+                            const float *inv_freq, int rot_dims, int interleaved, float magnitude, const int32_t *row_pos,
+                            const int32_t *row_seq, void *cache, int cache_dtype, const int32_t *page_table, int max_pages,
+                            int n_pages_total, int n_rows, int heads, int dim, int rot_dim, int rank, void *stream);
+int sb_head_product_gated(void *out, int out_dtype, int out_stride, int out_hstride, const void *in, int in_dtype,
+                          int in_stride, int in_hstride, const void *w, int w_dtype, const float *gate, int gate_stride,
+                          int gate_per_head, int n_rows, int heads, int n_in, int n_out, void *stream);
+int sb_head_product_gated_bf16(void *out, int out_stride, int out_hstride, const void *in, int in_stride, int in_hstride,
+                               const void *w, const float *gate, int gate_stride, int gate_per_head, int n_rows, int heads,
+                               int n_in, int n_out, void *stream);
+int sb_moe_route_grouped(int32_t *ids, float *weights, const float *z, int n_rows, int stride, int n_experts, int top,
+                         int has_gate, int score_kind, float score_scale, int n_groups, int keep_groups, void *stream);
+int sb_moe_router_grouped(int32_t *ids, float *weights, const void *h, int h_dtype, const float *w, int n_rows, int n_in,
+                          int n_experts, int top, int has_gate, int score_kind, float score_scale, int n_groups,
+                          int keep_groups, void *stream);
 
 #ifdef __cplusplus
 }

@@ -55,6 +55,13 @@ def _dev(*ts) -> None:
             raise KernelLibraryError("kernel operands must be contiguous")
 
 
+def _on_gpu(*ts) -> None:
+    """For operands that may be views of wider rows: on the GPU, layout checked by the caller."""
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise KernelLibraryError("kernel operands must live on the GPU (there is no CPU path)")
+
+
 def _i32(t: torch.Tensor, n: int, what: str) -> None:
     if t.dtype != torch.int32 or t.numel() < n:
         raise KernelLibraryError(f"{what} must be int32 with at least {n} elements")
@@ -190,7 +197,7 @@ def add_scaled(resid: torch.Tensor, y: torch.Tensor, scale: float) -> None:
     check(library.core().sb_add_scaled(_p(resid), _p(y), _dt(y), float(scale), resid.numel(), _stream()))
 
 
-ACTIVATIONS = {"silu": 1, "gelu_tanh": 2, "xielu": 3}      # sb_act of csrc/sb_hip.h
+ACTIVATIONS = {"silu": 1, "gelu_tanh": 2, "xielu": 3, "gelu_erf": 4, "relu_sq": 5}      # sb_act of csrc/sb_hip.h
 
 
 def activate(x: torch.Tensor, out_dtype: torch.dtype, activation: str, params: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -219,6 +226,50 @@ def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     return out
 
 
+def rmsnorm_pair(x: torch.Tensor, weight1: Optional[torch.Tensor], weight2: Optional[torch.Tensor], eps: float,
+                 out_dtype: torch.dtype, second: bool = True):
+    """Two RMS norms of the same float32 rows in one pass: (x inv) w1 and (x inv) w2 with one root mean
+    square for both.  ``x`` may be a view of wider rows (columns of a product's result): its last axis
+    dense, its rows any distance apart.  ``second`` false: the first alone (returns (y1, None))."""
+    _dev(weight1, weight2)
+    _on_gpu(x)
+    if x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1:
+        raise KernelLibraryError("the norm's input must be float32 [rows, width], dense along a row")
+    n, width = x.shape
+    for w in (weight1, weight2):
+        if w is not None and w.numel() != width:
+            raise KernelLibraryError(f"a norm weight has {w.numel()} elements, the rows have {width}")
+    if weight1 is not None and weight2 is not None and weight1.dtype != weight2.dtype:
+        raise KernelLibraryError("the two norm weights must be of one type")
+    wt = weight1 if weight1 is not None else weight2
+    y1 = torch.empty((n, width), dtype=out_dtype, device=x.device)
+    y2 = torch.empty((n, width), dtype=out_dtype, device=x.device) if second else None
+    check(library.core().sb_rmsnorm_pair(_p(y1), _p(y2), _DT[out_dtype], _p(x), x.stride(0) if n > 1 else width, _p(weight1),
+                                         _p(weight2), _dt(wt) if wt is not None else 0, n, width, float(eps), _stream()))
+    return y1, y2
+
+
+def sigmoid_mul_(x: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """x *= sigmoid(gate) in place, element by element: ``x`` [rows, width] dense, ``gate`` float32
+    [rows, width], possibly a view of wider rows."""
+    _dev(x)
+    _on_gpu(gate)
+    if x.dim() != 2 or not x.is_contiguous() or gate.dtype != torch.float32 or gate.shape != x.shape or gate.stride(1) != 1:
+        raise KernelLibraryError("sigmoid_mul_ takes dense rows and a float32 gate of the same shape")
+    n, width = x.shape
+    check(library.core().sb_sigmoid_mul(_p(x), _dt(x), _p(gate), gate.stride(0) if n > 1 else width, n, width, _stream()))
+    return x
+
+
+def softcap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x <- cap tanh(x / cap) in place (float32)."""
+    _dev(x)
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelLibraryError("softcap_ takes dense float32 values")
+    check(library.core().sb_softcap(_p(x), float(cap), x.numel(), _stream()))
+    return x
+
+
 def _check_cache(k_cache, v_cache, heads_kv, head_dim):
     if k_cache.dim() != 4 or v_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (heads_kv, PAGE, head_dim) \
             or tuple(v_cache.shape[1:]) != (heads_kv, head_dim, PAGE) or k_cache.shape[0] != v_cache.shape[0] \
@@ -239,19 +290,22 @@ def rope_kv_store(qkv: torch.Tensor, q_dtype: torch.dtype, inv_freq: Optional[to
                   freq_factors: Optional[torch.Tensor], rot_dims: int, row_pos: torch.Tensor,
                   row_seq: torch.Tensor, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
                   page_table: Optional[torch.Tensor], heads_q: int, heads_kv: int, head_dim: int,
-                  bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  bias: Optional[torch.Tensor] = None, v_dim: int = 0, magnitude: float = 1.0) -> torch.Tensor:
     """Rotate queries and keys of ``qkv`` [n, (hq+2hkv)*hd], return the queries
     [n, hq*hd] in ``q_dtype`` and store keys and values in the paged cache.
     ``heads_kv`` = 0 (and no cache) for a layer that stores nothing.  ``qkv`` may be
     [slices, n, width]: partial sums of the projection, added here in ascending order;
-    ``bias`` (float32 [width]) is added after them."""
+    ``bias`` (float32 [width]) is added after them.  ``v_dim``: the size of a value head when it
+    is not the keys' (the row is then [hq*hd | hkv*hd | hkv*v_dim]); ``magnitude`` multiplies every
+    cosine and sine."""
     _dev(qkv, inv_freq, freq_factors, row_pos, row_seq, k_cache, v_cache, page_table, bias)
     n_slices = 1
     if qkv.dim() == 3:
         n_slices = qkv.shape[0]
         qkv = qkv.view(-1, qkv.shape[2])
     n = qkv.shape[0] // n_slices
-    need = (heads_q + 2 * heads_kv) * head_dim
+    v_dim = int(v_dim) or head_dim
+    need = (heads_q + heads_kv) * head_dim + heads_kv * v_dim
     if qkv.dim() != 2 or qkv.shape[1] < need:
         raise KernelLibraryError(f"qkv rows have {qkv.shape[1]} elements, {need} are needed")
     if bias is not None and (bias.dtype != torch.float32 or bias.numel() < need):
@@ -264,15 +318,15 @@ def rope_kv_store(qkv: torch.Tensor, q_dtype: torch.dtype, inv_freq: Optional[to
     _i32(row_pos, n, "row positions")
     max_pages = n_pages = 0
     if heads_kv > 0:
-        _check_cache(k_cache, v_cache, heads_kv, head_dim)
+        _check_cache_kv(k_cache, v_cache, heads_kv, head_dim, v_dim)
         _check_rows(row_pos, row_seq, page_table, n)
         max_pages, n_pages = page_table.shape[1], k_cache.shape[0]
     q = torch.empty((n, heads_q * head_dim), dtype=q_dtype, device=qkv.device)
     lib = library.core()
-    check(lib.sb_rope_kv_store(
+    check(lib.sb_rope_kv_store_sized(
         _p(q), _dt(q), _p(qkv), _dt(qkv), qkv.shape[1], n_slices, _p(bias), _p(inv_freq), _p(freq_factors), rot_dims,
         _p(row_pos), _p(row_seq), _p(k_cache), _p(v_cache), _dt(k_cache) if k_cache is not None else 0,
-        _p(page_table), max_pages, n_pages, n, heads_q, heads_kv, head_dim, _stream()))
+        _p(page_table), max_pages, n_pages, n, heads_q, heads_kv, head_dim, v_dim, float(magnitude), _stream()))
     return q
 
 
@@ -901,16 +955,26 @@ def mingru_scan(p: torch.Tensor, state: torch.Tensor, cu_rows: torch.Tensor, slo
 def latent_prepare(p: torch.Tensor, q_off: int, kv_off: int, act_dtype: torch.dtype, c_weight: Optional[torch.Tensor],
                    eps: float, inv_freq: Optional[torch.Tensor], rot_dims: int, interleaved: bool,
                    row_pos: torch.Tensor, row_seq: torch.Tensor, cache: Optional[torch.Tensor],
-                   page_table: Optional[torch.Tensor], heads: int, dim: int, rot_dim: int, rank: int):
-    """A step's rows of a latent-attention layer's input product ``p`` float32 [rows, n]: returns
+                   page_table: Optional[torch.Tensor], heads: int, dim: int, rot_dim: int, rank: int,
+                   kv_rows: Optional[torch.Tensor] = None, magnitude: float = 1.0):
+    """``kv_rows`` float32 [rows, m] (a view of rows is fine): the rows that hold the latent's part at
+    ``kv_off`` when the queries come out of a product of their own (None: ``p``); ``magnitude``
+    multiplies every cosine and sine.  A step's rows of a latent-attention layer's input product ``p`` float32 [rows, n]: returns
     (q_plain [rows, heads, dim], q_latent [rows, heads, rank + rot_dim] whose last rot_dim numbers
     are the rotated query parts; the first rank are left for :func:`head_product`), and, with
     ``kv_off`` >= 0, stores the normed latent and the rotated key part of every row at its
     position in ``cache`` [pages, PAGE, rank + rot_dim]."""
     _dev(p, c_weight, inv_freq, row_pos, row_seq, cache, page_table)
+    _on_gpu(kv_rows)
     if p.dtype != torch.float32 or p.dim() != 2:
         raise KernelLibraryError("latent_prepare takes float32 rows")
     n, stride = p.shape
+    kv_stride = 0
+    if kv_rows is not None:
+        if kv_rows.dtype != torch.float32 or kv_rows.dim() != 2 or kv_rows.shape[0] != n or kv_rows.stride(1) != 1 \
+                or (kv_off >= 0 and kv_off + rank + rot_dim > kv_rows.shape[1]):
+            raise KernelLibraryError("the latent's rows must be float32 [rows, >= kv_off + rank + rot_dim]")
+        kv_stride = kv_rows.stride(0) if n > 1 else kv_rows.shape[1]
     latent = rank + rot_dim
     _i32(row_pos, n, "row positions")
     _i32(row_seq, n, "row sequences")
@@ -927,20 +991,21 @@ def latent_prepare(p: torch.Tensor, q_off: int, kv_off: int, act_dtype: torch.dt
         max_pages, n_pages = page_table.shape[1], cache.shape[0]
     q_plain = torch.empty((n, heads, dim), dtype=act_dtype, device=p.device)
     q_latent = torch.empty((n, heads, latent), dtype=act_dtype, device=p.device)
-    check(library.core().sb_latent_prepare(
-        _p(q_plain), _p(q_latent), _DT[act_dtype], _p(p), stride, int(q_off), int(kv_off), _p(c_weight),
-        _dt(c_weight) if c_weight is not None else 0, float(eps), _p(inv_freq), int(rot_dims), 1 if interleaved else 0,
-        _p(row_pos), _p(row_seq), _p(cache) if kv_off >= 0 else None, _dt(cache) if kv_off >= 0 else 0,
+    check(library.core().sb_latent_prepare_split(
+        _p(q_plain), _p(q_latent), _DT[act_dtype], _p(p), stride, int(q_off), _p(kv_rows), int(kv_stride), int(kv_off),
+        _p(c_weight), _dt(c_weight) if c_weight is not None else 0, float(eps), _p(inv_freq), int(rot_dims),
+        1 if interleaved else 0, float(magnitude), _p(row_pos), _p(row_seq), _p(cache) if kv_off >= 0 else None, _dt(cache) if kv_off >= 0 else 0,
         _p(page_table) if kv_off >= 0 else None, max_pages, n_pages, n, heads, dim, rot_dim, rank, _stream()))
     return q_plain, q_latent
 
 
 def head_product(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None,
-                 fast: bool = True) -> torch.Tensor:
+                 fast: bool = True, gate_per_head: bool = False) -> torch.Tensor:
     """out[t, a, :n_out] = w[a] x[t, a, :] for every head a: ``x`` [rows, heads, n_in] (a view
     whose last axis is dense), ``w`` [heads, n_out, n_in], ``out`` [rows, heads, >= n_out] (a view
     likewise; only the first n_out numbers of a head are written); ``gate`` float32 [rows, >= heads *
-    n_out] (a view of rows): the result times sigmoid(gate).  bfloat16 operands whose inner size and
+    n_out] (a view of rows): the result times sigmoid(gate); with ``gate_per_head`` the gate is [rows, >= heads],
+    one number for all outputs of a head.  bfloat16 operands whose inner size and
     strides are multiples of 8 run on the matrix cores (``fast``), the rest on the plain kernel."""
     for t in (x, w, out, gate):
         if t is not None and not t.is_cuda:
@@ -956,19 +1021,21 @@ def head_product(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Opti
         raise KernelLibraryError("head_product takes rows that are dense along their last axis, x and w of one type")
     g_stride = 0
     if gate is not None:
-        if gate.dtype != torch.float32 or gate.dim() != 2 or gate.shape[0] != rows or gate.shape[1] < heads * n_out \
-                or gate.stride(1) != 1:
-            raise KernelLibraryError("the gate must be float32 [rows, heads * out]")
+        if gate.dtype != torch.float32 or gate.dim() != 2 or gate.shape[0] != rows or gate.stride(1) != 1 \
+                or gate.shape[1] < (heads if gate_per_head else heads * n_out):
+            raise KernelLibraryError("the gate must be float32 [rows, heads * out] (or [rows, heads], a number a head)")
         g_stride = gate.stride(0)
     lib = library.core()
     if fast and x.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and x.data_ptr() % 16 == 0 \
             and w.data_ptr() % 16 == 0 and lib.sb_head_product_bf16_ok(out.stride(0), out.stride(1), x.stride(0),
                                                                        x.stride(1), n_in):
-        check(lib.sb_head_product_bf16(_p(out), out.stride(0), out.stride(1), _p(x), x.stride(0), x.stride(1), _p(w),
-                                       _p(gate), g_stride, rows, heads, n_in, n_out, _stream()))
+        check(lib.sb_head_product_gated_bf16(_p(out), out.stride(0), out.stride(1), _p(x), x.stride(0), x.stride(1), _p(w),
+                                             _p(gate), g_stride, 1 if gate_per_head else 0, rows, heads, n_in, n_out,
+                                             _stream()))
         return out
-    check(lib.sb_head_product(_p(out), _dt(out), out.stride(0), out.stride(1), _p(x), _dt(x), x.stride(0),
-                              x.stride(1), _p(w), _dt(w), _p(gate), g_stride, rows, heads, n_in, n_out, _stream()))
+    check(lib.sb_head_product_gated(_p(out), _dt(out), out.stride(0), out.stride(1), _p(x), _dt(x), x.stride(0),
+                                    x.stride(1), _p(w), _dt(w), _p(gate), g_stride, 1 if gate_per_head else 0, rows, heads,
+                                    n_in, n_out, _stream()))
     return out
 
 
@@ -1210,22 +1277,30 @@ def headnorm_kv_store(qkv: torch.Tensor, q_dtype: torch.dtype, q_weight: Optiona
 
 def attention_capped_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor,
                            row_pos: torch.Tensor, row_seq: torch.Tensor, heads_q: int, heads_kv: int, head_dim: int,
-                           v_dim: int, scale: float, window: int, softcap: float, sink: bool) -> torch.Tensor:
+                           v_dim: int, scale: float, window: int, softcap: float, sink: bool,
+                           sink_scores: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of rows ``q`` [n, hq*hd] over the cache by the plain kernel, values of ``v_dim``,
     scores capped as softcap tanh(s / softcap) (0: not), with ``sink`` one more key of score 0
-    without a value in every softmax; [n, hq*v_dim]."""
-    _dev(q, k_cache, v_cache, page_table, row_pos, row_seq)
+    without a value in every softmax (``sink_scores`` float32 [hq]: of the head's own score instead); [n, hq*v_dim]."""
+    _dev(q, k_cache, v_cache, page_table, row_pos, row_seq, sink_scores)
+    _check_sink(sink, sink_scores, heads_q)
     n = q.shape[0]
     if q.dim() != 2 or q.shape[1] != heads_q * head_dim:
         raise KernelLibraryError(f"queries must be [rows, {heads_q * head_dim}]")
     _check_cache_kv(k_cache, v_cache, heads_kv, head_dim, v_dim)
     _check_rows(row_pos, row_seq, page_table, n)
     out = torch.empty((n, heads_q * v_dim), dtype=q.dtype, device=q.device)
-    check(library.core().sb_attention_capped(
+    check(library.core().sb_attention_sink(
         _p(out), _p(q), _dt(q), q.shape[1], _p(k_cache), _p(v_cache), _dt(k_cache), _p(page_table),
         page_table.shape[1], k_cache.shape[0], _p(row_pos), _p(row_seq), n, heads_q, heads_kv, head_dim, v_dim,
-        float(scale), int(window), float(softcap), 1 if sink else 0, _stream()))
+        float(scale), int(window), float(softcap), 1 if sink else 0, _p(sink_scores), _stream()))
     return out
+
+
+def _check_sink(sink, sink_scores, heads_q):
+    if sink_scores is not None and (not sink or sink_scores.dtype != torch.float32 or sink_scores.numel() != heads_q
+                                    or not sink_scores.is_contiguous()):
+        raise KernelLibraryError(f"a sink's scores must be float32 [{heads_q}], of a sink that is switched on")
 
 
 def scale_(x: torch.Tensor, scale: float) -> torch.Tensor:
@@ -1287,15 +1362,25 @@ def moe_plan(ids: Optional[torch.Tensor], n_experts: int, n_pairs: Optional[int]
     return MoEPlan(ids, int(n_pairs), int(n_experts))
 
 
+def _expert_code(gated: bool, pair: str, single: Optional[str]) -> int:
+    """The `gated` argument of the experts' products."""
+    if gated:
+        if single is not None:
+            raise KernelLibraryError("a gated weight gives pairs; an activation of its own belongs to experts without a gate")
+        return EXPERT_PAIRS[pair]
+    return EXPERT_SINGLES[single] if single is not None else 0
+
+
 def moe_product(x: torch.Tensor, w: MoEWeight, plan: MoEPlan, x_div: int, out_dtype: torch.dtype,
-                limit: float = 0.0, alpha: float = 1.0, pair: str = "swish_clamp") -> torch.Tensor:
+                limit: float = 0.0, alpha: float = 1.0, pair: str = "swish_clamp", single: Optional[str] = None) -> torch.Tensor:
     """Y[p] = X[p // x_div] W_e^T for every pair p of ``plan``; a gated weight gives the pair of its
-    two halves that ``pair`` names (the clamped swish pair, or "silu": silu(g) u).  bfloat16 operands with an inner size in eights run on the matrix
+    two halves that ``pair`` names (the clamped swish pair, or "silu": silu(g) u); a weight without a gate
+    takes ``single``, the activation of every output ("relu_sq": max(z, 0)^2; None: the product as it is).  bfloat16 operands with an inner size in eights run on the matrix
     cores, the pairs grouped by expert on the device; everything else takes the plain kernel."""
     if w.experts != plan.n_experts:
         raise KernelLibraryError(f"the plan counts {plan.n_experts} experts, the weight has {w.experts}")
     if not (w.fast and x.dtype == torch.bfloat16 and w.w.dtype == torch.bfloat16 and w.n_in % 8 == 0):
-        return moe_product_plain(x, w.w, plan.ids, plan.n_pairs, x_div, out_dtype, w.gated, limit, alpha, pair)
+        return moe_product_plain(x, w.w, plan.ids, plan.n_pairs, x_div, out_dtype, w.gated, limit, alpha, pair, single)
     _dev(x)
     if x.dim() != 2 or x.shape[1] != w.n_in or (plan.n_pairs + x_div - 1) // x_div > x.shape[0]:
         raise KernelLibraryError(f"expert product shapes do not match: x {tuple(x.shape)}, w {tuple(w.w.shape)}, "
@@ -1304,21 +1389,22 @@ def moe_product(x: torch.Tensor, w: MoEWeight, plan: MoEPlan, x_div: int, out_dt
     y = torch.empty((plan.n_pairs, w.n_out), dtype=out_dtype, device=x.device)
     check(library.core().sb_moe_product_bf16(
         _p(y), _dt(y), _p(x), _p(w.w), _p(plan.order), _p(plan.tiles), _p(plan.n_tiles), plan.max_tiles, plan.tile_rows,
-        plan.n_pairs, int(x_div), w.n_out, w.n_in, EXPERT_PAIRS[pair] if w.gated else 0, float(limit), float(alpha), _stream()))
+        plan.n_pairs, int(x_div), w.n_out, w.n_in, _expert_code(w.gated, pair, single), float(limit), float(alpha), _stream()))
     return y
 
 
 def attention_capped(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor, ctx,
                      heads_q: int, heads_kv: int, head_dim: int, v_dim: int, scale: float, window: int,
-                     softcap: float, sink: bool, fast: bool = True) -> torch.Tensor:
+                     softcap: float, sink: bool, fast: bool = True, sink_scores: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of a step's rows over the cache with values of their own size, capped scores and a
     sink (see :func:`attention_capped_plain`).  bfloat16 with key and value sizes in steps of 16
     runs on the matrix cores; everything else takes the plain kernel."""
     if fast and capped_attention_mfma_ok(q.dtype, k_cache.dtype, head_dim, v_dim):
         return attention_capped_mfma(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_tiles(CAPPED_ROW_TILE),
-                                     heads_q, heads_kv, head_dim, v_dim, scale, window, softcap, sink)
+                                     heads_q, heads_kv, head_dim, v_dim, scale, window, softcap, sink,
+                                     sink_scores=sink_scores)
     return attention_capped_plain(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_seq, heads_q, heads_kv,
-                                  head_dim, v_dim, scale, window, softcap, sink)
+                                  head_dim, v_dim, scale, window, softcap, sink, sink_scores)
 
 
 CAPPED_ROW_TILE = 16        # rows of a run that a block of the matrix-core kernel takes (sb_cattn_tile_rows)
@@ -1333,11 +1419,12 @@ def capped_attention_mfma_ok(q_dtype, cache_dtype, head_dim: int, v_dim: int) ->
 def attention_capped_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor,
                           row_pos: torch.Tensor, tiles: torch.Tensor, heads_q: int, heads_kv: int, head_dim: int,
                           v_dim: int, scale: float, window: int, softcap: float, sink: bool,
-                          chunks: Optional[int] = None) -> torch.Tensor:
+                          chunks: Optional[int] = None, sink_scores: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The matrix-core form of :func:`attention_capped_plain`.  ``tiles`` int32 [n, 4]: the rows in
     runs of up to 16 consecutive rows of one sequence.  ``chunks``: over how many blocks a run's
     pages are shared out (None: chosen from the shapes alone, so that a recorded step replays)."""
-    _dev(q, k_cache, v_cache, page_table, row_pos, tiles)
+    _dev(q, k_cache, v_cache, page_table, row_pos, tiles, sink_scores)
+    _check_sink(sink, sink_scores, heads_q)
     n = q.shape[0]
     if q.dim() != 2 or q.shape[1] != heads_q * head_dim or q.dtype != torch.bfloat16:
         raise KernelLibraryError(f"queries must be bfloat16 [rows, {heads_q * head_dim}]")
@@ -1362,9 +1449,10 @@ def attention_capped_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
         part_ml = torch.empty((chunks, n, heads_q, 2), dtype=torch.float32, device=q.device)
     out = torch.empty((n, heads_q * v_dim), dtype=torch.bfloat16, device=q.device)
     lib = library.capped_attention_library(head_dim, v_dim)
-    check(lib.sb_cattn_bf16(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(page_table), max_pages, k_cache.shape[0],
-                            _p(row_pos), _p(tiles), n_tiles, n, heads_q, heads_kv, float(scale), int(window),
-                            float(softcap), 1 if sink else 0, chunks, chunk_pages, _p(part_o), _p(part_ml), _stream()),
+    check(lib.sb_cattn_sink_bf16(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(page_table), max_pages, k_cache.shape[0],
+                                 _p(row_pos), _p(tiles), n_tiles, n, heads_q, heads_kv, float(scale), int(window),
+                                 float(softcap), 1 if sink else 0, chunks, chunk_pages, _p(part_o), _p(part_ml), None, None, 0,
+                                 _p(sink_scores), _stream()),
           lib, "sb_cattn_last_error")
     return out
 
@@ -1373,25 +1461,29 @@ def moe_max_top() -> int:
     return int(library.core().sb_moe_max_top())
 
 
-def moe_route(z: torch.Tensor, n_experts: int, top: int, has_gate: bool, score: str = "softmax_chosen", score_scale: float = 1.0):
+def moe_route(z: torch.Tensor, n_experts: int, top: int, has_gate: bool, score: str = "softmax_chosen", score_scale: float = 1.0,
+              groups: int = 1, keep_groups: int = 1):
     """From router scores ``z`` float32 [n, >= n_experts (+ 1)]: the ``top`` largest of the first
     ``n_experts`` of every row (ties to the lower number) as int32 [n, top], and float32 [n, top + 1]:
     the softmax over the chosen scores, then sigmoid(z[:, n_experts]) with ``has_gate`` (else 0).
     ``score`` "sigmoid": the scores are sigmoid(z), the largest are chosen and their weights are those
-    scores times ``score_scale``, not renormalized."""
+    scores times ``score_scale``, not renormalized; "softmax_all": the same with the softmax of z over
+    all experts as scores.  ``groups`` > 1: the experts lie in that many equal groups of neighbours, a
+    group's score is its best expert's, and only experts of the ``keep_groups`` best groups are chosen."""
     _dev(z)
     if z.dtype != torch.float32 or z.dim() != 2:
         raise KernelLibraryError("router scores must be float32 [rows, experts]")
     n = z.shape[0]
     ids = torch.empty((n, top), dtype=torch.int32, device=z.device)
     weights = torch.empty((n, top + 1), dtype=torch.float32, device=z.device)
-    check(library.core().sb_moe_route_scored(_p(ids), _p(weights), _p(z), n, z.shape[1], int(n_experts), int(top),
-                                             1 if has_gate else 0, ROUTER_SCORES[score], float(score_scale), _stream()))
+    check(library.core().sb_moe_route_grouped(_p(ids), _p(weights), _p(z), n, z.shape[1], int(n_experts), int(top),
+                                              1 if has_gate else 0, ROUTER_SCORES[score], float(score_scale), int(groups),
+                                              int(keep_groups), _stream()))
     return ids, weights
 
 
 def moe_router(h: torch.Tensor, w: torch.Tensor, n_experts: int, top: int, has_gate: bool, score: str = "softmax_chosen",
-               score_scale: float = 1.0):
+               score_scale: float = 1.0, groups: int = 1, keep_groups: int = 1):
     """The router in one launch: z = h w^T in float32 (``w`` float32 [n_experts (+ 1 with
     ``has_gate``), width], ``h`` rows of either type), then what :func:`moe_route` gives."""
     _dev(h, w)
@@ -1401,8 +1493,9 @@ def moe_router(h: torch.Tensor, w: torch.Tensor, n_experts: int, top: int, has_g
     n = h.shape[0]
     ids = torch.empty((n, top), dtype=torch.int32, device=h.device)
     weights = torch.empty((n, top + 1), dtype=torch.float32, device=h.device)
-    check(library.core().sb_moe_router_scored(_p(ids), _p(weights), _p(h), _dt(h), _p(w), n, h.shape[1], int(n_experts),
-                                              int(top), 1 if has_gate else 0, ROUTER_SCORES[score], float(score_scale), _stream()))
+    check(library.core().sb_moe_router_grouped(_p(ids), _p(weights), _p(h), _dt(h), _p(w), n, h.shape[1], int(n_experts),
+                                               int(top), 1 if has_gate else 0, ROUTER_SCORES[score], float(score_scale),
+                                               int(groups), int(keep_groups), _stream()))
     return ids, weights
 
 
@@ -1419,7 +1512,7 @@ def swish_clamp_mul(gu: torch.Tensor, out_dtype: torch.dtype, limit: float, alph
 
 def moe_product_plain(x: torch.Tensor, w: torch.Tensor, ids: Optional[torch.Tensor], n_pairs: int, x_div: int,
                       out_dtype: torch.dtype, gated: bool = False, limit: float = 0.0, alpha: float = 1.0,
-                      pair: str = "swish_clamp") -> torch.Tensor:
+                      pair: str = "swish_clamp", single: Optional[str] = None) -> torch.Tensor:
     """Y[p] = X[p // x_div] W_e^T, e = ids[p] (None: expert 0), by the plain kernel.  ``w``
     [experts, out (or 2*out, gate over up, with ``gated``), in]; gated: the clamped swish pair
     g' sigmoid(alpha g') (u' + 1) with g' = min(g, limit), u' = u cut to +-limit."""
@@ -1434,13 +1527,15 @@ def moe_product_plain(x: torch.Tensor, w: torch.Tensor, ids: Optional[torch.Tens
         raise KernelLibraryError("more pairs than rows to take them from")
     y = torch.empty((n_pairs, n_out), dtype=out_dtype, device=x.device)
     check(library.core().sb_moe_product(_p(y), _dt(y), _p(x), _dt(x), _p(w), _dt(w), _p(ids), n_pairs, int(x_div),
-                                        n_out, n_in, n_experts, EXPERT_PAIRS[pair] if gated else 0, float(limit), float(alpha), _stream()))
+                                        n_out, n_in, n_experts, _expert_code(gated, pair, single), float(limit), float(alpha),
+                                        _stream()))
     return y
 
 
 # ---- short convolutions over time, recurrences with a matrix state, attention with shared weights ----
-ROUTER_SCORES = {"softmax_chosen": 0, "sigmoid": 1}      # score_kind of sb_moe_route_scored
-EXPERT_PAIRS = {"swish_clamp": 1, "silu": 2}             # `gated` of the experts' products
+ROUTER_SCORES = {"softmax_chosen": 0, "sigmoid": 1, "softmax_all": 2}      # score_kind of sb_moe_route_grouped
+EXPERT_PAIRS = {"swish_clamp": 1, "silu": 2}             # `gated` of the experts' products: pairs of a gate and an up row
+EXPERT_SINGLES = {"relu_sq": 3}                          # the same argument for experts without a gate: one row an output
 
 
 def time_conv_max_taps() -> int:

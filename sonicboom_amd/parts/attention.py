@@ -15,7 +15,10 @@ Every size and switch is a parameter of the spec:
     sink (one more key of score 0 without a value in every softmax: the weights are
     exp(s_j) / (1 + sum exp(s_j))), value_mix ("first": the values of this step's rows are kept
     for later layers under ``value_mix_key``; "mix": v <- (1 - lam) v + lam v_first with the layer's
-    own number lam; what is mixed is what the cache keeps)
+    own number lam; what is mixed is what the cache keeps), sink_scores (the sink's score is a number of
+    the query head's own, a tensor of heads_q numbers, as it is: weights exp(s_j) / (exp(sink_a) + sum
+    exp(s_j))), out_gate (the heads' results side by side times sigmoid(W_g h), number by number, before
+    the output product; W_g is stacked under q, k and v)
 
 and the position encoding is a nested part.  The three input projections are
 packed into one matrix when the mixer is built, so a step runs one product
@@ -37,7 +40,8 @@ from .spec import PartSpec, TensorSpec
 
 NAMES = {"q_weight": "q_proj.weight", "k_weight": "k_proj.weight", "v_weight": "v_proj.weight",
          "o_weight": "o_proj.weight", "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias",
-         "o_bias": "o_proj.bias", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "value_mix": "value_mix"}
+         "o_bias": "o_proj.bias", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight", "value_mix": "value_mix",
+         "sink": "sink", "g_weight": "g"}
 
 
 def attention_spec(prefix: str, width: int, heads_q: int, heads_kv: int, head_dim: int,
@@ -45,7 +49,8 @@ def attention_spec(prefix: str, width: int, heads_q: int, heads_kv: int, head_di
                    qkv_bias: bool = True, out_bias: bool = False, out_scale: float = 1.0,
                    v_dim: Optional[int] = None, qk_norm: bool = False, qk_norm_eps: float = 0.0,
                    softcap: float = 0.0, sink: bool = False, value_mix: Optional[str] = None,
-                   value_mix_key: str = "values", names: Optional[dict] = None) -> PartSpec:
+                   value_mix_key: str = "values", names: Optional[dict] = None, sink_scores: bool = False,
+                   out_gate: bool = False) -> PartSpec:
     """``names``: what the file calls a role's tensor after ``prefix``, where that is not what
     ``NAMES`` says."""
     nm = dict(NAMES, **(names or {}))
@@ -66,6 +71,12 @@ def attention_spec(prefix: str, width: int, heads_q: int, heads_kv: int, head_di
     if qk_norm:
         tensors["q_norm"] = TensorSpec(prefix + nm["q_norm"], (head_dim,), init=(1.0, 0.02))
         tensors["k_norm"] = TensorSpec(prefix + nm["k_norm"], (head_dim,), init=(1.0, 0.02))
+    if sink_scores:
+        if not sink:
+            raise ValueError("scores of a sink belong to a mixer that has one")
+        tensors["sink"] = TensorSpec(prefix + nm["sink"], (heads_q,), init=(0.0, 0.5))
+    if out_gate:
+        tensors["g_weight"] = TensorSpec(prefix + nm["g_weight"], (heads_q * v_dim, width))
     if value_mix not in (None, "first", "mix"):
         raise ValueError(f"value_mix is None, 'first' or 'mix', not {value_mix!r}")
     if value_mix is not None:
@@ -76,6 +87,7 @@ def attention_spec(prefix: str, width: int, heads_q: int, heads_kv: int, head_di
         "window": int(window), "scale": scale, "qkv_bias": qkv_bias, "out_bias": out_bias,
         "out_scale": float(out_scale), "v_dim": v_dim, "qk_norm": bool(qk_norm), "qk_norm_eps": float(qk_norm_eps),
         "softcap": float(softcap), "sink": bool(sink), "value_mix": value_mix, "value_mix_key": value_mix_key,
+        "sink_scores": bool(sink_scores), "out_gate": bool(out_gate),
     }, tensors, {"position": position})
 
 
@@ -108,27 +120,38 @@ class Attention(Mixer):
         self.value_mix = p.get("value_mix")
         self.value_mix_key = p.get("value_mix_key", "values")
         self.lam = tensors.get("value_mix") if self.value_mix == "mix" else None
-        # head norms, capped scores, a sink, values of their own size or mixed values: the path whose
-        # kernels take them (no rotation there)
-        self.extended = bool(self.qk_norm or self.softcap or self.sink or self.value_mix or self.v_dim != self.head_dim)
+        self.sink_scores = tensors["sink"].float().contiguous() if p.get("sink_scores") else None
+        self.out_gate = bool(p.get("out_gate", False))
+        # head norms, capped scores, a sink, values of their own size or mixed values, an output gate: the path
+        # whose kernels take them.  Head norms and mixed values go with mixers that do not rotate (one kernel
+        # norms, mixes and stores); the others rotate and store with the kernel of the plain path.
+        self.extended = bool(self.qk_norm or self.softcap or self.sink or self.value_mix or self.v_dim != self.head_dim
+                             or self.out_gate)
+        self.head_norm_path = bool(self.qk_norm or self.value_mix)
         if self.extended:
-            if self.position.rotary_tables() != (None, None, 0):
-                raise ValueError("head norms, capped scores, sinks and values of their own size are built for "
-                                 "mixers without a rotation")
-            if p.get("qkv_bias", True):
-                raise ValueError("head norms, capped scores, sinks and values of their own size are built for "
-                                 "mixers without biases on q, k and v")
+            if self.head_norm_path and self.position.rotary_tables() != (None, None, 0):
+                raise ValueError("head norms and mixed values are built for mixers without a rotation")
+            if self.position.rotary_tables() is None:
+                raise ValueError("capped scores, sinks, gates and values of their own size take a rotary position "
+                                 "encoding, or none")
+            if self.head_norm_path and p.get("qkv_bias", True):
+                raise ValueError("head norms and mixed values are built for mixers without biases on q, k and v")
         if rt.fast_kernels and not self.extended:
             # (groups of one and two heads per kv head take higher tiles on the matrix cores)
             self.row_tile = ops.attention_row_tiles(self.heads_q, self.heads_kv, self.head_dim, rt.act_dtype)
 
         ws = [tensors["q_weight"], tensors["k_weight"], tensors["v_weight"]]
+        self.g_off = sum(int(w.shape[0]) for w in ws)        # where the output gate's columns start in the stacked product
+        if self.out_gate:
+            ws.append(tensors["g_weight"])
         w_qkv = torch.cat(ws, dim=0) if all(w.dtype == ws[0].dtype for w in ws) \
             else torch.cat([w.float() for w in ws], dim=0)
         b_qkv = None
         if p.get("qkv_bias", True):
             bs = [tensors["q_bias"], tensors["k_bias"], tensors["v_bias"]]
             b_qkv = torch.cat([b.float() for b in bs], dim=0)
+            if self.out_gate:
+                b_qkv = torch.cat([b_qkv, torch.zeros(tensors["g_weight"].shape[0], dtype=torch.float32, device=b_qkv.device)])
         self.qkv = Linear(w_qkv, b_qkv, rt.fast_kernels)
         # an order entry that reads another entry's cache projects queries only: the model asks for
         # that projection (query_only) before finish_build() drops the separate query weight
@@ -167,7 +190,34 @@ class Attention(Mixer):
             raise ValueError("a mixer that hands its result over has no multiplier of its own")
         return self.out.raw(self._attend(h, ctx, binding))
 
+    def _attend_rotating(self, h, ctx, binding):
+        """The extended path of mixers that rotate (or have no position encoding and no head norms): the plain path's
+        rotate-and-store kernel with the values' own size, attention with the sink's scores, the output gate."""
+        rt = self.rt
+        if not binding.writes_cache:
+            raise RuntimeError("this mixer stores the keys and values it reads")
+        # (with a gate the product is taken whole: the gate's columns are read where they lie)
+        qkv = None if self.out_gate else self.qkv.partial(h)
+        bias = None
+        if qkv is not None:
+            bias = self.qkv.bias
+        else:
+            qkv = self.qkv(h, torch.float32)
+        inv_freq, freq_factors, rot_dims = self.position.rotary_tables()
+        page_table = ctx.page_table(binding.group)
+        q = ops.rope_kv_store(qkv, rt.act_dtype, inv_freq, freq_factors, rot_dims, ctx.row_pos, ctx.row_seq,
+                              binding.k_cache, binding.v_cache, page_table, self.heads_q, self.heads_kv, self.head_dim,
+                              bias=bias, v_dim=self.v_dim, magnitude=float(getattr(self.position, "magnitude", 1.0)))
+        a = ops.attention_capped(q, binding.k_cache, binding.v_cache, page_table, ctx, self.heads_q, self.heads_kv,
+                                 self.head_dim, self.v_dim, self.scale, self.window, self.softcap, self.sink,
+                                 fast=rt.fast_kernels, sink_scores=self.sink_scores)
+        if self.out_gate:
+            ops.sigmoid_mul_(a, qkv[:, self.g_off:self.g_off + self.heads_q * self.v_dim])
+        return a
+
     def _attend_extended(self, h, ctx, binding):
+        if not self.head_norm_path:
+            return self._attend_rotating(h, ctx, binding)
         rt = self.rt
         writes = binding.writes_cache
         if not writes:
@@ -192,7 +242,7 @@ class Attention(Mixer):
                                   self.head_dim, self.v_dim, store=writes, v_first=v_first, lam=self.lam, v_out=v_out)
         return ops.attention_capped(q, binding.k_cache, binding.v_cache, page_table, ctx, self.heads_q, self.heads_kv,
                                     self.head_dim, self.v_dim, self.scale, self.window, self.softcap, self.sink,
-                                    fast=rt.fast_kernels)
+                                    fast=rt.fast_kernels, sink_scores=self.sink_scores)
 
     def _attend(self, h, ctx, binding):
         """The heads' results [rows, heads_q * v_dim] in the activation type; keys and values of the

@@ -14,6 +14,11 @@ input_taps - 1 inputs are per-sequence state of the block.
 x += norm(mixer(x)); x += norm(ffn(x)).  The mixer and the feed-forward hand their result over
 (``produce``) and one pass sums its slices, norms it, adds it into the stream and leaves the new
 stream in the activation type for the sublayer that reads it next.
+
+``parallel``: both sublayers read the same stream, each through a norm of its own, and their results
+join it together: x += mixer(norm1(x)) + ffn(norm2(x)).  One pass norms the stream for both (the root
+mean square is the same, the weights differ); the mixer and the feed-forward then add into the stream
+one after the other.
 """
 from __future__ import annotations
 
@@ -165,3 +170,65 @@ class OutNormBlock(Part):
         if trace is not None:
             trace("after_ffn", x)
         return h
+
+
+def parallel_block_spec(mixer_norm: PartSpec, mixer: PartSpec, ffn_norm: PartSpec = None, ffn: PartSpec = None) -> PartSpec:
+    parts = {"mixer_norm": mixer_norm, "mixer": mixer}
+    if ffn is not None:
+        if ffn_norm is None:
+            raise ValueError("a block with a feed-forward needs the norm before it")
+        parts.update(ffn_norm=ffn_norm, ffn=ffn)
+    return PartSpec("block", "parallel", {}, {}, parts)
+
+
+@register_part("block", "parallel")
+class ParallelBlock(Part):
+    category = "block"
+
+    def __init__(self, spec, tensors, parts, rt):
+        super().__init__(spec, tensors, parts, rt)
+        self.mixer_norm = parts["mixer_norm"]
+        self.mixer = parts["mixer"]
+        self.ffn_norm = parts.get("ffn_norm")
+        self.ffn = parts.get("ffn")              # None: the block is its mixer's branch alone
+        # with two branches the block norms for both in one pass of its own; alone, the mixer's norm is what
+        # the block before may apply in its last pass
+        self.first_norm = self.mixer_norm if self.ffn is None else None
+        a, b = self.mixer_norm, self.ffn_norm
+        # one pass for both norms when they are RMS norms over whole rows with the same eps and plain weights
+        self.one_pass = b is not None and all(
+            getattr(n, "fusable", False) and getattr(n, "groups", 1) == 1 and hasattr(n, "eps") for n in (a, b)) \
+            and a.eps == b.eps and (a.weight is None) == (b.weight is None) \
+            and (a.weight is None or a.weight.dtype == b.weight.dtype)
+
+    def forward(self, x, ctx, binding, h=None, next_norm=None):
+        """Run the block on the residual stream ``x`` in place.  ``h`` is mixer_norm(x) when the block
+        before has already computed it.  Returns next_norm(x) when the last pass produced it, else None.
+        Both branches are normed before either result joins the stream."""
+        act = self.rt.act_dtype
+        f = None
+        if self.ffn is not None:
+            if h is None and self.one_pass:
+                h, f = ops.rmsnorm_pair(x, self.mixer_norm.weight, self.ffn_norm.weight, self.mixer_norm.eps, act)
+            else:
+                f = self.ffn_norm.forward(x, act)
+        if h is None:
+            h = self.mixer_norm.forward(x, act)
+        last = self.ffn is None
+        if getattr(self.mixer, "fuses_norm", False):
+            out = self.mixer.forward(h, x, ctx, binding, then_norm=next_norm if last else None)
+        else:
+            out = self.mixer.forward(h, x, ctx, binding)
+        trace = getattr(ctx, "trace", None)
+        if trace is not None:
+            trace("after_mixer", x)
+        if last:
+            return out
+        out = None
+        if getattr(self.ffn, "fuses_norm", False):
+            out = self.ffn.forward(f, x, ctx, then_norm=next_norm)
+        else:
+            self.ffn.forward(f, x, ctx)
+        if trace is not None:
+            trace("after_ffn", x)
+        return out

@@ -20,9 +20,10 @@ def embedding_spec(name: str, vocab: int, width: int) -> PartSpec:
                     {"table": TensorSpec(name, (vocab, width))})
 
 
-def head_spec(name: str, vocab: int, width: int, scale: float = 1.0) -> PartSpec:
-    """``name`` may be the embedding table's name: the head then shares it.  ``scale`` multiplies the logits."""
-    return PartSpec("head", "linear", {"vocab": vocab, "width": width, "scale": float(scale)},
+def head_spec(name: str, vocab: int, width: int, scale: float = 1.0, softcap: float = 0.0) -> PartSpec:
+    """``name`` may be the embedding table's name: the head then shares it.  ``scale`` multiplies the logits;
+    ``softcap`` > 0: they then become softcap * tanh(logits / softcap)."""
+    return PartSpec("head", "linear", {"vocab": vocab, "width": width, "scale": float(scale), "softcap": float(softcap)},
                     {"weight": TensorSpec(name, (vocab, width))})
 
 
@@ -90,7 +91,12 @@ class LinearHead(Part):
         self.proj = Linear(tensors["weight"], None, rt.fast_kernels)
         self.vocab = int(spec.params["vocab"])
         self.scale = float(spec.params.get("scale", 1.0))
+        self.softcap = float(spec.params.get("softcap", 0.0) or 0.0)
+        if self.softcap < 0:
+            raise ValueError("the logits' cap must not be negative")
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         logits = self.proj(h, torch.float32)
-        return logits if self.scale == 1.0 else ops.scale_(logits, self.scale)
+        if self.scale != 1.0:
+            logits = ops.scale_(logits, self.scale)
+        return ops.softcap_(logits, self.softcap) if self.softcap else logits

@@ -10,7 +10,8 @@ are stacked into one [2*inner, width] matrix when the part is built, so a
 step runs one product for both; its float32 result feeds the activation
 kernel, whose output is rounded once to the activation type.
 
-``dense``: y = W_down act(W_up f), the activation one of ``ops.ACTIVATIONS``; "xielu" reads its two
+``dense``: y = W_down act(W_up f + b_up) + b_down (biases when the spec names them), the activation one
+of ``ops.ACTIVATIONS`` ("gelu_erf": z Phi(z) by the error function; "relu_sq": max(z, 0)^2); "xielu" reads its two
 numbers (p, q) from a tensor of the layer: softplus(p) z^2 + z/2 for z > 0 and
 (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2 else.  The up product leaves in float32, the activation
 kernel rounds once to the activation type.
@@ -76,11 +77,17 @@ class GatedDenseFFN(Part):
 
 
 def dense_ffn_spec(up_name: str, down_name: str, width: int, inner: int, activation: str,
-                   act_name: str = None, out_scale: float = 1.0) -> PartSpec:
-    """``act_name``: the tensor that holds the activation's numbers (xIELU's two)."""
+                   act_name: str = None, out_scale: float = 1.0, up_bias_name: str = None,
+                   down_bias_name: str = None) -> PartSpec:
+    """``act_name``: the tensor that holds the activation's numbers (xIELU's two); ``up_bias_name``,
+    ``down_bias_name``: the biases of the two products, for feed-forwards that have them."""
     tensors = {"up_weight": TensorSpec(up_name, (inner, width)), "down_weight": TensorSpec(down_name, (width, inner))}
     if act_name is not None:
         tensors["act_params"] = TensorSpec(act_name, (2,), init=(0.0, 0.5))
+    if up_bias_name is not None:
+        tensors["up_bias"] = TensorSpec(up_bias_name, (inner,), init=(0.0, 0.02))
+    if down_bias_name is not None:
+        tensors["down_bias"] = TensorSpec(down_bias_name, (width,), init=(0.0, 0.02))
     return PartSpec("ffn", "dense", {"width": width, "inner": inner, "activation": activation,
                                      "out_scale": float(out_scale)}, tensors)
 
@@ -99,15 +106,16 @@ class DenseFFN(Part):
         self.act_params = tensors.get("act_params")
         if self.activation == "xielu" and self.act_params is None:
             raise ValueError("xIELU needs the tensor with its two numbers")
-        self.up = Linear(tensors["up_weight"], None, rt.fast_kernels)
-        self.down = Linear(tensors["down_weight"], None, rt.fast_kernels)
+        up_b, down_b = tensors.get("up_bias"), tensors.get("down_bias")
+        self.up = Linear(tensors["up_weight"], None if up_b is None else up_b.float(), rt.fast_kernels)
+        self.down = Linear(tensors["down_weight"], None if down_b is None else down_b.float(), rt.fast_kernels)
         self.out_scale = float(p.get("out_scale", 1.0))
 
     fuses_norm = True
     graph_safe = True     # its launches depend on device buffers only
 
     def forward(self, h, x, ctx, then_norm=None):
-        """x += out_scale * W_down act(W_up h).  Returns then_norm(x) when the down projection could
+        """x += out_scale * (W_down act(W_up h + b_up) + b_down).  Returns then_norm(x) when the down projection could
         apply the norm in its last pass, else None."""
         mid = ops.activate(self.up(h, torch.float32), self.rt.act_dtype, self.activation, self.act_params)
         return self.down.add_into(mid, x, then_norm, self.rt.act_dtype, scale=self.out_scale)

@@ -11,6 +11,11 @@ reference writes it and handed to the kernel as a table.
 ``rot_dims`` numbers, pair i turning by position * base^(-2i / rot_dims); for mixers whose
 kernels take the pairing as an argument.
 
+Both rotary kinds take, in place of the base, a table of the pairs' frequencies (``frequencies``:
+the angle of pair i at position p is p times entry i) and a ``magnitude`` that multiplies every
+cosine and sine; :func:`stretched_frequencies` makes both for frequencies divided by a factor, all
+alike ("linear") or only the slow ones with a ramp between two wavelengths ("ramp").
+
 ``none``: no encoding.
 """
 from __future__ import annotations
@@ -26,11 +31,48 @@ from .spec import PartSpec
 
 
 def rope_spec(head_dim: int, base: float, rot_dims: int = 0,
-              freq_factors: Optional[Sequence[float]] = None, score_scale: float = 1.0) -> PartSpec:
+              freq_factors: Optional[Sequence[float]] = None, score_scale: float = 1.0,
+              frequencies: Optional[Sequence[float]] = None, magnitude: float = 1.0) -> PartSpec:
+    """``frequencies``: the pairs' frequencies themselves (one per rotated pair), in place of base^(-2i/n)."""
     return PartSpec("position", "rope", {
         "head_dim": head_dim, "base": float(base), "rot_dims": int(rot_dims),
         "freq_factors": None if freq_factors is None else [float(f) for f in freq_factors],
-        "score_scale": float(score_scale)})
+        "score_scale": float(score_scale),
+        "frequencies": None if frequencies is None else [float(f) for f in frequencies], "magnitude": float(magnitude)})
+
+
+def stretched_frequencies(dims: int, base: float, kind: Optional[str] = None, factor: float = 1.0, original: float = 0.0,
+                          fast: float = 32.0, slow: float = 1.0):
+    """(frequencies of the dims / 2 pairs, magnitude) for f_i = base^(-2i/dims) stretched by ``factor``:
+
+    * ``kind`` None: f_i as they are;
+    * "linear": every f_i / factor;
+    * "ramp": pair i keeps the share 1 - r_i of f_i and takes r_i of f_i / factor, r_i rising from 0 to 1 between
+      the pair that makes ``fast`` turns over ``original`` positions and the one that makes ``slow`` (their places
+      d(t) = dims ln(original / (2 pi t)) / (2 ln base), the lower rounded down and not below 0, the upper rounded
+      up and not above dims - 1, at least 0.001 apart); cosines and sines grow by 0.1 ln(factor) + 1.
+
+    Everything in float64; the kernels round each frequency once to float32."""
+    half = dims // 2
+    f = [float(base) ** (-2.0 * i / dims) for i in range(half)]
+    if kind is None:
+        return f, 1.0
+    if factor <= 0:
+        raise ValueError("a rotation is stretched by a positive factor")
+    if kind == "linear":
+        return [v / factor for v in f], 1.0
+    if kind != "ramp":
+        raise ValueError(f"unknown kind of stretched rotation {kind!r}")
+
+    def place(turns):
+        return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+    lo = max(math.floor(place(fast)), 0)
+    hi = min(math.ceil(place(slow)), dims - 1)
+    out = []
+    for i, v in enumerate(f):
+        r = min(1.0, max(0.0, (i - lo) / max(hi - lo, 0.001)))
+        out.append(v / factor * r + v * (1.0 - r))
+    return out, 0.1 * math.log(factor) + 1.0
 
 
 def scaled_rope_tables(kind: str, factor: float, head_dim: int, base: float, original_ctx: int,
@@ -69,14 +111,28 @@ def scaled_rope_tables(kind: str, factor: float, head_dim: int, base: float, ori
     return table, score
 
 
-def rope_interleaved_spec(rot_dims: int, base: float) -> PartSpec:
-    return PartSpec("position", "rope_interleaved", {"rot_dims": int(rot_dims), "base": float(base)})
+def rope_interleaved_spec(rot_dims: int, base: float, frequencies: Optional[Sequence[float]] = None,
+                          magnitude: float = 1.0) -> PartSpec:
+    return PartSpec("position", "rope_interleaved", {
+        "rot_dims": int(rot_dims), "base": float(base),
+        "frequencies": None if frequencies is None else [float(f) for f in frequencies], "magnitude": float(magnitude)})
+
+
+def _given_frequencies(params, rot_dims: int, default):
+    """The spec's own table of frequencies rounded once to float32, or ``default``."""
+    given = params.get("frequencies")
+    if given is None:
+        return default
+    if len(given) != rot_dims // 2:
+        raise ValueError(f"{len(given)} frequencies for {rot_dims // 2} rotated pairs")
+    return np.asarray(given, dtype=np.float64).astype(np.float32)
 
 
 class Position(Part):
     category = "position"
     score_scale = 1.0
     interleaved = False     # rotary encodings: pairs are (i, i + rot_dims / 2); True: (2i, 2i + 1)
+    magnitude = 1.0         # rotary encodings: what every cosine and sine is multiplied by
 
     def rotary_tables(self):
         """(inv_freq, freq_factors, rot_dims) for the fused rotate-and-store
@@ -112,6 +168,8 @@ class Rope(Position):
         i = np.arange(n // 2, dtype=np.float32)
         expo = (np.float32(-2.0) * i / np.float32(n)).astype(np.float32)
         inv = np.exp((expo * log_base).astype(np.float32)).astype(np.float32)
+        inv = _given_frequencies(p, n, inv)
+        self.magnitude = float(p.get("magnitude", 1.0) or 1.0)
         self.inv_freq = torch.from_numpy(inv).to(rt.device)
         ff = p.get("freq_factors")
         self.freq_factors = None
@@ -138,6 +196,8 @@ class RopeInterleaved(Position):
         base = float(spec.params["base"])
         i = np.arange(self.rot_dims // 2, dtype=np.float64)
         inv = np.power(np.float64(base), -2.0 * i / max(self.rot_dims, 1)).astype(np.float32)
+        inv = _given_frequencies(spec.params, self.rot_dims, inv)
+        self.magnitude = float(spec.params.get("magnitude", 1.0) or 1.0)
         self.inv_freq = torch.from_numpy(inv).to(rt.device) if self.rot_dims else None
 
     def rotary_tables(self):
