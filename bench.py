@@ -36,7 +36,9 @@ one prompt step and one decode step with what it reaches of its roofline (bytes 
 8 TB/s, or flops over the dense bf16 peak, whichever is the larger time).  A table goes to standard
 error, one JSON line to standard output.  ``--design tatelorn`` puts the Tatelorn design (blocks that
 norm what their sublayers give back, attention with head norms, capped scores and a sink, routed
-experts) in the Rasizen design's place (``--design nalasun``: the Nalasun design, state-space and delta-rule
+experts) in the Rasizen design's place (``--design fitatar``: the Fitatar design, layers of two parallel branches with
+latent attention through a query latent, gated attention with a sink score a head and experts chosen within groups;
+``--design nalasun``: the Nalasun design, state-space and delta-rule
 recurrences, attention with shared head weights and routed experts behind short convolutions): eight layers, the first with a dense gated feed-forward, the
 others with eight experts of which a row takes two plus a shared one, so that a row passes as many
 feed-forward weights as in the Qwen2.5 design beside it, and the same heads.
@@ -263,8 +265,10 @@ def main() -> int:
     ap.add_argument("--prompt", type=int, default=PROMPT, help="cached prompt tokens per sequence")
     ap.add_argument("--context", type=int, default=CONTEXT, help="cache size per sequence")
     ap.add_argument("--workload", choices=("steady", "mixed", "forms", "designs"), default="steady")
-    ap.add_argument("--design", choices=("rasizen", "tatelorn", "nalasun"), default="rasizen",
+    ap.add_argument("--design", choices=("rasizen", "tatelorn", "nalasun", "fitatar"), default="rasizen",
                     help="--workload designs: the design that runs beside the Qwen2.5 design")
+    ap.add_argument("--beside", choices=("qwen2", "rasizen", "tatelorn", "nalasun", "fitatar"), default="qwen2",
+                    help="--workload designs: the design at the same sizes that the first one runs beside")
     ap.add_argument("--design-sizes", default="2048,4096",
                     help="--workload designs: the widths of the layer sizes to run, comma separated")
     ap.add_argument("--batches", default="1,8", help="--workload forms: the batch sizes, comma separated")
@@ -711,6 +715,33 @@ def nalasun_sizes(width, vocab=32768, experts=8, top=2):
             "canon": {"taps": 3}, "layers": layers}
 
 
+def fitatar_sizes(width, vocab=32768, experts=8, top=2):
+    """Layer sizes in the manner of a real model of this width, eight layers: latent attention with heads of 128
+    plain + 64 rotated numbers and 128 values, a latent of 512 and a query latent of half a width (the first keeps
+    its latent, the fifth reads it), attention with heads of 128 for keys and values, a quarter of them kv heads;
+    the first layer with a dense feed-forward of 4 widths, the others with `experts` experts of one width in four
+    groups of which a row takes `top` from the best three, and a shared expert of 2 widths: a row passes as many
+    feed-forward weights as in the Qwen2.5 layer beside it."""
+    heads = width // 128
+    rot = {"base": 1e6, "dims": 64, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    lat = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "q_rank": max(256, width // 2),
+           "scale": 192 ** -0.5, "rot": rot}
+    att = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+           "rot": {"base": 1e6, "dims": 128, "scaling": {"factor": 8.0}}}
+    routed = {"kind": "moe", "router": {"experts": experts, "top": top, "groups": {"count": 4, "keep": 3}},
+              "expert": {"ff": width}, "shared": {"ff": 2 * width}}
+    layers = []
+    for i in range(8):
+        if i == 0:
+            layers.append({"type": "latent_attention", "mixer": dict(lat), "mlp": {"kind": "dense", "ff": 4 * width}})
+        elif i == 4:
+            layers.append({"type": "latent_attention", "mixer": dict(lat, kv_from=0), "mlp": routed})
+        else:
+            layers.append({"type": "attention", "mixer": dict(att), "mlp": routed})
+    return {"architecture": "Fitatar", "vocab": vocab, "width": width, "embedding": {"scale": 0.5}, "logit_softcap": 30.0,
+            "norm": {"eps": 1e-6}, "layers": layers}
+
+
 VECTOR_F32_FLOPS = 157.3e12      # the vector units' float32 peak, against which the recurrences' scans are priced
 
 
@@ -757,6 +788,8 @@ class AllOpsTimer:
                         label = f"{_name} {tuple(args[1].shape)}"
                     elif _name == "time_conv":
                         label = f"{_name} {args[1].shape[0]}"
+                    elif _name in ("activate", "sigmoid_mul_", "rmsnorm_pair"):
+                        label = f"{_name} {args[0].shape[-1]}"
                     elif _name == "moe_product":
                         label = f"{_name} {args[1].experts}x{args[1].n_out}x{args[1].n_in}{' gated' if args[1].gated else ''}"
                     self.records.append((label, e0, e1))
@@ -802,6 +835,14 @@ def design_roofline(label, us, calls, rows, depth, batch, width, cfgs):
         nbytes = rows * cfgs["gru"] * (12 + 2)
     elif label == "activate":
         nbytes = rows * cfgs["ff"] * (4 + 2)
+    elif label.startswith("activate "):
+        nbytes = rows * int(label.split()[1]) * (4 + 2)
+    elif label.startswith("sigmoid_mul_ "):
+        nbytes = rows * int(label.split()[1]) * (2 + 2 + 4)
+    elif label.startswith("rmsnorm_pair "):
+        nbytes = rows * int(label.split()[1]) * (4 + 2 + (2 if int(label.split()[1]) == width else 0))
+    elif label == "softcap_":
+        nbytes = (rows if decode else 1) * cfgs["vocab"] * 8
     elif label == "latent_prepare":
         nbytes = rows * (4 * (H * 192 + rank + rot) + 2 * (H * (192 + rank) + rank + rot))
     elif label.startswith("head_product"):
@@ -865,9 +906,9 @@ def design_comparison(a) -> int:
     rng = np.random.default_rng(0)
     out, table = {}, []
     for width in (int(v) for v in a.design_sizes.split(",")):
-        beside = {"rasizen": rasizen_sizes, "tatelorn": tatelorn_sizes, "nalasun": nalasun_sizes}[a.design]
-        beside = (a.design, beside(width))
-        for design, cfg in (beside, ("qwen2", qwen_sizes(width))):
+        sizes = {"rasizen": rasizen_sizes, "tatelorn": tatelorn_sizes, "nalasun": nalasun_sizes, "fitatar": fitatar_sizes,
+                 "qwen2": qwen_sizes}
+        for design, cfg in ((a.design, sizes[a.design](width)), (a.beside, sizes[a.beside](width))):
             model = DecoderModel.from_random(cfg, seed=0, dtype="bfloat16", device="cuda:0")
             heads = width // 128
             cfgs = {"heads": heads, "rank": 512, "rot": 64, "window": 4096 if design == "rasizen" else 1 << 30,
@@ -929,7 +970,7 @@ def design_comparison(a) -> int:
     for key, v in out.items():
         print(f"RESULT {key} prefill_tokens_per_s={v['prefill_tokens_per_s']} decode_tokens_per_s={v['decode_tokens_per_s']} "
               f"prefill_ms={v['prefill_ms']} decode_step_ms={v['decode_step_ms']}", file=sys.stderr)
-    print(json.dumps({"workload": "designs", "design": a.design, "prompt": a.prompt, "batch": a.batch, "steps": a.steps, "dtype": "bf16",
+    print(json.dumps({"workload": "designs", "design": a.design, "beside": a.beside, "prompt": a.prompt, "batch": a.batch, "steps": a.steps, "dtype": "bf16",
                       "data": "synthetic", "models": out}))
     return 0
 

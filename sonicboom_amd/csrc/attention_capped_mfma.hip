@@ -68,6 +68,7 @@ struct Args {
   const float *dist_r1, *dist_r2;      // [heads_q] or NULL: the bias by the distance's logarithm
   int all_values;                      // 1: blockIdx.y also counts the kv head whose values are read
   const float *sink_scores;            // [heads_q] or NULL: the sink's score a head (NULL: 0)
+  const float *gate; int gate_stride;  // [rows, gate_stride] or NULL: the result times sigmoid(gate[row][h * DV + d])
   unsigned round_blocks;       // blocks the GPU takes one of per CU
 };
 
@@ -299,9 +300,15 @@ __global__ void __launch_bounds__(kThreads) capped_attention_kernel(Args a) {
     bf16_t *dst = a.out + (size_t(row) * out_heads + (a.all_values ? h * a.heads_kv + vh : h)) * DV;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
+      float r[4] = {o[dt][0] * inv, o[dt][1] * inv, o[dt][2] * inv, o[dt][3] * inv};
+      if (a.gate) {
+        const float *gp = a.gate + size_t(row) * a.gate_stride + size_t(h) * DV + 16 * dt + 4 * g;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] = r[i] * (1.0f / (1.0f + expf(-gp[i])));
+      }
       uint2 w;
-      w.x = pack_bf16(o[dt][0] * inv, o[dt][1] * inv);
-      w.y = pack_bf16(o[dt][2] * inv, o[dt][3] * inv);
+      w.x = pack_bf16(r[0], r[1]);
+      w.y = pack_bf16(r[2], r[3]);
       *reinterpret_cast<uint2 *>(dst + 16 * dt + 4 * g) = w;
     }
   } else {
@@ -324,7 +331,7 @@ constexpr int kMergeAtOnce = 16;
 
 __global__ void __launch_bounds__(256)
 merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o, const float *__restrict__ part_ml, int chunks,
-             size_t n_heads /* rows * heads_q */) {
+             size_t n_heads /* rows * heads_q */, const float *__restrict__ gate, int gate_stride, int heads_q) {
   const size_t idx = size_t(blockIdx.x) * 256 + threadIdx.x;
   if (idx >= n_heads * DV) return;
   const size_t rh = idx / DV;
@@ -355,7 +362,12 @@ merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o, const f
       den = fmaf(w, lc[i], den);
     }
   }
-  out[idx] = f32_to_bf16(den > 0.0f ? num / den : 0.0f);
+  float r = den > 0.0f ? num / den : 0.0f;
+  if (gate) {
+    const size_t row = rh / heads_q;
+    r = r * (1.0f / (1.0f + expf(-gate[row * gate_stride + (idx - row * heads_q * DV)])));
+  }
+  out[idx] = f32_to_bf16(r);
 }
 
 }  // namespace
@@ -389,7 +401,7 @@ extern "C" int sb_cattn_sink_bf16(void *out, const void *q, const void *k_cache,
                                   const int32_t *tiles, int n_tiles, int n_rows, int heads_q, int heads_kv, float scale,
                                   int window, float softcap, int sink, int chunks, int chunk_pages, float *part_o,
                                   float *part_ml, const float *dist_r1, const float *dist_r2, int all_values,
-                                  const float *sink_scores, void *stream);
+                                  const float *sink_scores, const float *gate, int gate_stride, void *stream);
 
 // The same with the bias r1[h] ln(1 + r2[h] distance) taken off every score (dist_r1, dist_r2 f32 [heads_q], or both
 // NULL) and, with all_values, every query head's weights applied to the values of every kv head: out bf16
@@ -402,18 +414,20 @@ extern "C" int sb_cattn_shared_bf16(void *out, const void *q, const void *k_cach
                                     void *stream) {
   return sb_cattn_sink_bf16(out, q, k_cache, v_cache, page_table, max_pages, n_pages, row_pos, tiles, n_tiles, n_rows, heads_q,
                             heads_kv, scale, window, softcap, sink, chunks, chunk_pages, part_o, part_ml, dist_r1, dist_r2,
-                            all_values, nullptr, stream);
+                            all_values, nullptr, nullptr, 0, stream);
 }
 
 // The same with a sink whose score is a number of the query head's own (sink_scores f32 [heads_q], as it is: not
-// scaled, not capped; NULL: 0).
+// scaled, not capped; NULL: 0), and with an output gate (f32 [rows, gate_stride] or NULL; not with all_values): the
+// result times sigmoid(gate[row * gate_stride + h * dv + d]).
 extern "C" int sb_cattn_sink_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
                                   const int32_t *page_table, int max_pages, int n_pages, const int32_t *row_pos,
                                   const int32_t *tiles, int n_tiles, int n_rows, int heads_q, int heads_kv, float scale,
                                   int window, float softcap, int sink, int chunks, int chunk_pages, float *part_o,
                                   float *part_ml, const float *dist_r1, const float *dist_r2, int all_values,
-                                  const float *sink_scores, void *stream) {
+                                  const float *sink_scores, const float *gate, int gate_stride, void *stream) {
   SB_REQUIRE(!sink_scores || sink, "sb_cattn_bf16: scores of a sink that is switched off");
+  SB_REQUIRE(!gate || (!all_values && gate_stride >= heads_q * DV), "sb_cattn_bf16: the gate's rows of %d are too short", gate_stride);
   SB_REQUIRE((dist_r1 == nullptr) == (dist_r2 == nullptr), "sb_cattn_bf16: the distance bias needs both of its numbers");
   SB_REQUIRE(out && q && k_cache && v_cache && page_table && row_pos && tiles, "sb_cattn_bf16: null pointer");
   SB_REQUIRE(n_tiles >= 0 && n_rows >= 0 && heads_q > 0 && heads_kv > 0 && max_pages > 0 && n_pages > 0 && window >= 0,
@@ -439,11 +453,12 @@ extern "C" int sb_cattn_sink_bf16(void *out, const void *q, const void *k_cache,
   a.round_blocks = unsigned(sb::cu_count());
   a.dist_r1 = dist_r1; a.dist_r2 = dist_r2; a.all_values = all_values ? 1 : 0;
   a.sink_scores = sink_scores;
+  a.gate = chunks == 1 ? gate : nullptr; a.gate_stride = gate_stride;      // (partial results are gated when they are merged)
   capped_attention_kernel<<<dim3(n_tiles, heads_kv * zgroups * value_heads, chunks), kThreads, 0, s>>>(a);
   int st = sb::check_launch("sb_cattn_bf16");
   if (st != SB_OK || chunks == 1) return st;
   const size_t n = size_t(n_rows) * heads_q * value_heads * DV;
   merge_kernel<<<unsigned((n + 255) / 256), 256, 0, s>>>((bf16_t *)out, part_o, part_ml, chunks,
-                                                         size_t(n_rows) * heads_q * value_heads);
+                                                         size_t(n_rows) * heads_q * value_heads, gate, gate_stride, heads_q);
   return sb::check_launch("sb_cattn_merge");
 }

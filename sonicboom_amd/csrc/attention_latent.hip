@@ -76,8 +76,8 @@ latent_prepare_kernel(TA *__restrict__ q_plain, TA *__restrict__ q_latent, const
         pair_index(j, rot_dims, interleaved, i0, i1);
         const float a = fpos * inv_freq[j];
         float y0, y1;
-        rotate_pair(r[i0], r[i1], magnitude == 1.0f ? cosf(a) : cosf(a) * magnitude,
-                    magnitude == 1.0f ? sinf(a) : sinf(a) * magnitude, y0, y1);
+        if (magnitude == 1.0f) rotate_pair(r[i0], r[i1], cosf(a), sinf(a), y0, y1);
+        else rotate_pair(r[i0], r[i1], cosf(a) * magnitude, sinf(a) * magnitude, y0, y1);
         st_f(dst, rank + i0, y0);
         st_f(dst, rank + i1, y1);
       }
@@ -100,8 +100,8 @@ latent_prepare_kernel(TA *__restrict__ q_plain, TA *__restrict__ q_latent, const
     const float *qr = q + a * hd + dim;
     const float ang = fpos * inv_freq[j];
     float y0, y1;
-    rotate_pair(qr[i0], qr[i1], magnitude == 1.0f ? cosf(ang) : cosf(ang) * magnitude,
-                magnitude == 1.0f ? sinf(ang) : sinf(ang) * magnitude, y0, y1);
+    if (magnitude == 1.0f) rotate_pair(qr[i0], qr[i1], cosf(ang), sinf(ang), y0, y1);
+    else rotate_pair(qr[i0], qr[i1], cosf(ang) * magnitude, sinf(ang) * magnitude, y0, y1);
     TA *dst = q_latent + (size_t(row) * heads + a) * latent + rank;
     st_f(dst, i0, y0);
     st_f(dst, i1, y1);

@@ -29,7 +29,8 @@ attention_plain_kernel(TA *__restrict__ out, const TA *__restrict__ q, int q_str
                        const int32_t *__restrict__ page_table, int max_pages, int n_pages_total,
                        const int32_t *__restrict__ row_pos, const int32_t *__restrict__ row_seq,
                        int heads_q, int heads_kv, int head_dim, float scale, int window, int v_dim,
-                       float softcap, int sink, const float *__restrict__ sink_scores) {
+                       float softcap, int sink, const float *__restrict__ sink_scores,
+                       const float *__restrict__ gate, int gate_stride) {
   __shared__ float qs[kMaxHeadDim];
   __shared__ float ps[64];
   const int row = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -84,7 +85,12 @@ attention_plain_kernel(TA *__restrict__ out, const TA *__restrict__ q, int q_str
 #pragma unroll
   for (int i = 0; i < kMaxHeadDim / 64; ++i) {
     const int d = lane + 64 * i;
-    if (d < v_dim) st_f(out, size_t(row) * heads_q * v_dim + size_t(h) * v_dim + d, o[i] * inv);
+    if (d < v_dim) {
+      float r = o[i] * inv;
+      // an output gate: the result times the sigmoid of the gate's number at the same place of the row
+      if (gate) r = r * (1.0f / (1.0f + expf(-gate[size_t(row) * gate_stride + size_t(h) * v_dim + d])));
+      st_f(out, size_t(row) * heads_q * v_dim + size_t(h) * v_dim + d, r);
+    }
   }
 }
 
@@ -116,7 +122,7 @@ extern "C" int sb_attention_sink(void *out, const void *q, int act_dtype, int q_
                                  int max_pages, int n_pages_total, const int32_t *row_pos,
                                  const int32_t *row_seq, int n_rows, int heads_q, int heads_kv,
                                  int head_dim, int v_dim, float scale, int window, float softcap, int sink,
-                                 const float *sink_scores, void *stream);
+                                 const float *sink_scores, const float *gate, int gate_stride, void *stream);
 
 extern "C" int sb_attention_capped(void *out, const void *q, int act_dtype, int q_stride, const void *k_cache,
                                    const void *v_cache, int cache_dtype, const int32_t *page_table,
@@ -126,18 +132,20 @@ extern "C" int sb_attention_capped(void *out, const void *q, int act_dtype, int 
                                    void *stream) {
   return sb_attention_sink(out, q, act_dtype, q_stride, k_cache, v_cache, cache_dtype, page_table, max_pages, n_pages_total,
                            row_pos, row_seq, n_rows, heads_q, heads_kv, head_dim, v_dim, scale, window, softcap, sink,
-                           nullptr, stream);
+                           nullptr, nullptr, 0, stream);
 }
 
 // The same with a sink whose score is a number of the query head's own, sink_scores f32 [heads_q]
-// (NULL: 0): weights exp(s_j) / (exp(sink_h) + sum exp(s_j)).
+// (NULL: 0): weights exp(s_j) / (exp(sink_h) + sum exp(s_j)); and with an output gate (or NULL): the
+// result [rows, heads_q * v_dim] times sigmoid(gate[row * gate_stride + i]), number by number.
 extern "C" int sb_attention_sink(void *out, const void *q, int act_dtype, int q_stride, const void *k_cache,
                                  const void *v_cache, int cache_dtype, const int32_t *page_table,
                                  int max_pages, int n_pages_total, const int32_t *row_pos,
                                  const int32_t *row_seq, int n_rows, int heads_q, int heads_kv,
                                  int head_dim, int v_dim, float scale, int window, float softcap, int sink,
-                                 const float *sink_scores, void *stream) {
+                                 const float *sink_scores, const float *gate, int gate_stride, void *stream) {
   SB_REQUIRE(!sink_scores || sink, "sb_attention: scores of a sink that is switched off");
+  SB_REQUIRE(!gate || gate_stride >= heads_q * v_dim, "sb_attention: the gate's rows of %d are too short", gate_stride);
   SB_REQUIRE(out && q && k_cache && v_cache && page_table && row_pos && row_seq,
              "sb_attention: null pointer");
   SB_REQUIRE(n_rows >= 0 && heads_q > 0 && heads_kv > 0 && head_dim > 0 && max_pages > 0 &&
@@ -160,7 +168,7 @@ extern "C" int sb_attention_sink(void *out, const void *q, int act_dtype, int q_
   attention_plain_kernel<TA, TC><<<grid, 64, 0, s>>>(                                            \
       (TA *)out, (const TA *)q, q_stride, (const TC *)k_cache, (const TC *)v_cache, page_table,  \
       max_pages, n_pages_total, row_pos, row_seq, heads_q, heads_kv, head_dim, scale, window, v_dim,  \
-      softcap, sink, sink_scores)
+      softcap, sink, sink_scores, gate, gate_stride)
   if (act_dtype == SB_F32 && cache_dtype == SB_F32) SB_GO(float, float);
   else if (act_dtype == SB_BF16 && cache_dtype == SB_BF16) SB_GO(bf16_t, bf16_t);
   else if (act_dtype == SB_F32 && cache_dtype == SB_BF16) SB_GO(float, bf16_t);

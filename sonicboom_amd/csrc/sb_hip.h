@@ -486,7 +486,8 @@ int sb_random_normal(void *out, int out_kind, uint64_t n, uint64_t first, uint64
  *   the rows x_stride apart (parts of wider rows).
  * sb_sigmoid_mul: x[t, i] *= sigmoid(gate[t * gate_stride + i]).  sb_softcap: x <- cap tanh(x / cap).
  * sb_rope_kv_store_sized: value heads of v_dim numbers; every cosine and sine times `magnitude`.
- * sb_attention_sink: the sink's score a number of the query head's own (sink_scores f32 [heads_q]).
+ * sb_attention_sink: the sink's score a number of the query head's own (sink_scores f32 [heads_q]); an output
+ *   gate, the result times sigmoid(gate[row * gate_stride + i]).
  * sb_latent_prepare_split: the latent's part read from rows of its own; `magnitude` as above.
  * sb_head_product_gated(_bf16): gate_per_head, one gate number a head.
  * sb_moe_route_grouped / sb_moe_router_grouped: score_kind 0 softmax over the chosen, 1 sigmoid, 2 softmax
@@ -505,7 +506,8 @@ int sb_rope_kv_store_sized(void *q_out, int q_dtype, const void *qkv, int qkv_dt
 int sb_attention_sink(void *out, const void *q, int act_dtype, int q_stride, const void *k_cache, const void *v_cache,
                       int cache_dtype, const int32_t *page_table, int max_pages, int n_pages_total,
                       const int32_t *row_pos, const int32_t *row_seq, int n_rows, int heads_q, int heads_kv, int head_dim,
-                      int v_dim, float scale, int window, float softcap, int sink, const float *sink_scores, void *stream);
+                      int v_dim, float scale, int window, float softcap, int sink, const float *sink_scores,
+                      const float *gate, int gate_stride, void *stream);
 int sb_latent_prepare_split(void *q_plain, void *q_latent, int act_dtype, const float *p, int row_stride, int q_off,
                             const float *kv_rows, int kv_stride, int kv_off, const void *c_weight, int c_w_dtype, float eps,
                             const float *inv_freq, int rot_dims, int interleaved, float magnitude, const int32_t *row_pos,

@@ -1278,12 +1278,14 @@ def headnorm_kv_store(qkv: torch.Tensor, q_dtype: torch.dtype, q_weight: Optiona
 def attention_capped_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor,
                            row_pos: torch.Tensor, row_seq: torch.Tensor, heads_q: int, heads_kv: int, head_dim: int,
                            v_dim: int, scale: float, window: int, softcap: float, sink: bool,
-                           sink_scores: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           sink_scores: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of rows ``q`` [n, hq*hd] over the cache by the plain kernel, values of ``v_dim``,
     scores capped as softcap tanh(s / softcap) (0: not), with ``sink`` one more key of score 0
-    without a value in every softmax (``sink_scores`` float32 [hq]: of the head's own score instead); [n, hq*v_dim]."""
+    without a value in every softmax (``sink_scores`` float32 [hq]: of the head's own score instead); [n, hq*v_dim].
+    ``gate`` float32 [n, hq*v_dim] (a view of wider rows is fine): the result times sigmoid(gate)."""
     _dev(q, k_cache, v_cache, page_table, row_pos, row_seq, sink_scores)
     _check_sink(sink, sink_scores, heads_q)
+    g_stride = _check_gate(gate, q.shape[0], heads_q * v_dim)
     n = q.shape[0]
     if q.dim() != 2 or q.shape[1] != heads_q * head_dim:
         raise KernelLibraryError(f"queries must be [rows, {heads_q * head_dim}]")
@@ -1293,8 +1295,18 @@ def attention_capped_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torc
     check(library.core().sb_attention_sink(
         _p(out), _p(q), _dt(q), q.shape[1], _p(k_cache), _p(v_cache), _dt(k_cache), _p(page_table),
         page_table.shape[1], k_cache.shape[0], _p(row_pos), _p(row_seq), n, heads_q, heads_kv, head_dim, v_dim,
-        float(scale), int(window), float(softcap), 1 if sink else 0, _p(sink_scores), _stream()))
+        float(scale), int(window), float(softcap), 1 if sink else 0, _p(sink_scores), _p(gate), g_stride, _stream()))
     return out
+
+
+def _check_gate(gate, rows, width) -> int:
+    """The distance between the rows of an output gate (0 without one)."""
+    if gate is None:
+        return 0
+    _on_gpu(gate)
+    if gate.dtype != torch.float32 or gate.dim() != 2 or tuple(gate.shape) != (rows, width) or gate.stride(1) != 1:
+        raise KernelLibraryError(f"an output gate must be float32 [{rows}, {width}], dense along a row")
+    return gate.stride(0) if rows > 1 else width
 
 
 def _check_sink(sink, sink_scores, heads_q):
@@ -1395,16 +1407,17 @@ def moe_product(x: torch.Tensor, w: MoEWeight, plan: MoEPlan, x_div: int, out_dt
 
 def attention_capped(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor, ctx,
                      heads_q: int, heads_kv: int, head_dim: int, v_dim: int, scale: float, window: int,
-                     softcap: float, sink: bool, fast: bool = True, sink_scores: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     softcap: float, sink: bool, fast: bool = True, sink_scores: Optional[torch.Tensor] = None,
+                     gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of a step's rows over the cache with values of their own size, capped scores and a
     sink (see :func:`attention_capped_plain`).  bfloat16 with key and value sizes in steps of 16
     runs on the matrix cores; everything else takes the plain kernel."""
     if fast and capped_attention_mfma_ok(q.dtype, k_cache.dtype, head_dim, v_dim):
         return attention_capped_mfma(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_tiles(CAPPED_ROW_TILE),
                                      heads_q, heads_kv, head_dim, v_dim, scale, window, softcap, sink,
-                                     sink_scores=sink_scores)
+                                     sink_scores=sink_scores, gate=gate)
     return attention_capped_plain(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_seq, heads_q, heads_kv,
-                                  head_dim, v_dim, scale, window, softcap, sink, sink_scores)
+                                  head_dim, v_dim, scale, window, softcap, sink, sink_scores, gate)
 
 
 CAPPED_ROW_TILE = 16        # rows of a run that a block of the matrix-core kernel takes (sb_cattn_tile_rows)
@@ -1419,13 +1432,15 @@ def capped_attention_mfma_ok(q_dtype, cache_dtype, head_dim: int, v_dim: int) ->
 def attention_capped_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor,
                           row_pos: torch.Tensor, tiles: torch.Tensor, heads_q: int, heads_kv: int, head_dim: int,
                           v_dim: int, scale: float, window: int, softcap: float, sink: bool,
-                          chunks: Optional[int] = None, sink_scores: Optional[torch.Tensor] = None) -> torch.Tensor:
+                          chunks: Optional[int] = None, sink_scores: Optional[torch.Tensor] = None,
+                          gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The matrix-core form of :func:`attention_capped_plain`.  ``tiles`` int32 [n, 4]: the rows in
     runs of up to 16 consecutive rows of one sequence.  ``chunks``: over how many blocks a run's
     pages are shared out (None: chosen from the shapes alone, so that a recorded step replays)."""
     _dev(q, k_cache, v_cache, page_table, row_pos, tiles, sink_scores)
     _check_sink(sink, sink_scores, heads_q)
     n = q.shape[0]
+    g_stride = _check_gate(gate, n, heads_q * v_dim)
     if q.dim() != 2 or q.shape[1] != heads_q * head_dim or q.dtype != torch.bfloat16:
         raise KernelLibraryError(f"queries must be bfloat16 [rows, {heads_q * head_dim}]")
     _check_cache_kv(k_cache, v_cache, heads_kv, head_dim, v_dim)
@@ -1452,7 +1467,7 @@ def attention_capped_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch
     check(lib.sb_cattn_sink_bf16(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(page_table), max_pages, k_cache.shape[0],
                                  _p(row_pos), _p(tiles), n_tiles, n, heads_q, heads_kv, float(scale), int(window),
                                  float(softcap), 1 if sink else 0, chunks, chunk_pages, _p(part_o), _p(part_ml), None, None, 0,
-                                 _p(sink_scores), _stream()),
+                                 _p(sink_scores), _p(gate), g_stride, _stream()),
           lib, "sb_cattn_last_error")
     return out
 

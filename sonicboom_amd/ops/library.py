@@ -89,7 +89,7 @@ _CORE_SIGNATURES = {
     "sb_softcap": [_P, _F, _Z, _P],
     "sb_rope_kv_store_sized": [_P, _I, _P, _I, _I, _I, _P, _P, _P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F,
                                _P],
-    "sb_attention_sink": [_P, _P, _I, _I, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _I, _P, _P],
+    "sb_attention_sink": [_P, _P, _I, _I, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _I, _P, _P, _I, _P],
     "sb_latent_prepare_split": [_P, _P, _I, _P, _I, _I, _P, _I, _I, _P, _I, _F, _P, _I, _I, _F, _P, _P, _P, _I, _P, _I, _I,
                                 _I, _I, _I, _I, _I, _P],
     "sb_head_product_gated": [_P, _I, _I, _I, _P, _I, _I, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
@@ -135,9 +135,9 @@ _CAPPED_ATTN_SIGNATURES = {
     "sb_cattn_bf16": [_P, _P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _F, _I, _I, _I, _P, _P, _P],
     # the same, then dist_r1, dist_r2, all_values, stream
     "sb_cattn_shared_bf16": [_P, _P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _F, _I, _I, _I, _P, _P, _P, _P, _I, _P],
-    # the same, then sink_scores, stream
+    # the same, then sink_scores, gate, gate_stride, stream
     "sb_cattn_sink_bf16": [_P, _P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _F, _I, _I, _I, _P, _P, _P, _P, _I, _P,
-                           _P],
+                           _P, _I, _P],
     "sb_cattn_tile_rows": [],
     "sb_cattn_key_dim": [],
     "sb_cattn_value_dim": [],

@@ -208,11 +208,11 @@ class Attention(Mixer):
         q = ops.rope_kv_store(qkv, rt.act_dtype, inv_freq, freq_factors, rot_dims, ctx.row_pos, ctx.row_seq,
                               binding.k_cache, binding.v_cache, page_table, self.heads_q, self.heads_kv, self.head_dim,
                               bias=bias, v_dim=self.v_dim, magnitude=float(getattr(self.position, "magnitude", 1.0)))
+        # the gate rides in the attention kernel's last pass (or, when a row's pages are shared out, in the merge)
+        gate = qkv[:, self.g_off:self.g_off + self.heads_q * self.v_dim] if self.out_gate else None
         a = ops.attention_capped(q, binding.k_cache, binding.v_cache, page_table, ctx, self.heads_q, self.heads_kv,
                                  self.head_dim, self.v_dim, self.scale, self.window, self.softcap, self.sink,
-                                 fast=rt.fast_kernels, sink_scores=self.sink_scores)
-        if self.out_gate:
-            ops.sigmoid_mul_(a, qkv[:, self.g_off:self.g_off + self.heads_q * self.v_dim])
+                                 fast=rt.fast_kernels, sink_scores=self.sink_scores, gate=gate)
         return a
 
     def _attend_extended(self, h, ctx, binding):

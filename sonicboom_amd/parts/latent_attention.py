@@ -38,18 +38,18 @@ def latent_attention_spec(prefix: str, width: int, heads: int, dim: int, rot_dim
                           gate_per_head: bool = False) -> PartSpec:
     """Tensors ``<prefix>q`` (or, with ``q_rank``, ``dq``, ``dq.norm`` and ``uq``), ``g``, ``o``, ``uk``, ``uv`` and,
     with ``own_latent``, ``dkv`` and ``dkv.norm``."""
-    tensors = {
+    if q_rank:
+        tensors = {"dq_weight": TensorSpec(prefix + "dq", (q_rank, width)),
+                   "dq_norm": TensorSpec(prefix + "dq.norm", (q_rank,), init=(1.0, 0.02)),
+                   "uq_weight": TensorSpec(prefix + "uq", (heads * (dim + rot_dim), q_rank))}
+    else:
+        tensors = {"q_weight": TensorSpec(prefix + "q", (heads * (dim + rot_dim), width))}
+    tensors.update({
         "uk_weight": TensorSpec(prefix + "uk", (heads * dim, kv_rank)),
         "uv_weight": TensorSpec(prefix + "uv", (heads * vdim, kv_rank)),
         "g_weight": TensorSpec(prefix + "g", (heads if gate_per_head else heads * vdim, width)),
         "o_weight": TensorSpec(prefix + "o", (width, heads * vdim)),
-    }
-    if q_rank:
-        tensors["dq_weight"] = TensorSpec(prefix + "dq", (q_rank, width))
-        tensors["dq_norm"] = TensorSpec(prefix + "dq.norm", (q_rank,), init=(1.0, 0.02))
-        tensors["uq_weight"] = TensorSpec(prefix + "uq", (heads * (dim + rot_dim), q_rank))
-    else:
-        tensors["q_weight"] = TensorSpec(prefix + "q", (heads * (dim + rot_dim), width))
+    })
     if own_latent:
         tensors["dkv_weight"] = TensorSpec(prefix + "dkv", (kv_rank + rot_dim, width))
         tensors["dkv_norm"] = TensorSpec(prefix + "dkv.norm", (kv_rank,), init=(1.0, 0.02))
