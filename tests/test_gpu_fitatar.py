@@ -100,14 +100,14 @@ def coded_routers(cfg, w):
     return w
 
 
-def sharpen(cfg, w, coded=True):
+def sharpen(cfg, w, coded=True, qk_gain=10.0):
     """Random N(0, 0.02) weights give flat scores, gates at one half and activations in their linear part.  Scale
     the projections so that scores spread over several units, gates move and the activations bend."""
     out = {}
     for name, a in w.items():
         a = np.array(a, dtype=np.float64)
         if name.endswith((".mix.q", ".mix.k", ".mix.dq", ".mix.uq", ".mix.dkv", ".mix.uk")):
-            a = a * 10.0
+            a = a * qk_gain
         elif name.endswith((".mix.v", ".mix.uv", ".mix.o", ".mix.g")):
             a = a * 8.0
         elif name.endswith((".up", ".down", ".sg")):
@@ -126,13 +126,13 @@ def sharpen(cfg, w, coded=True):
     return coded_routers(cfg, out) if coded else out
 
 
-def make_folder(tmp_path_factory, name, cfg, seed, coded=True):
+def make_folder(tmp_path_factory, name, cfg, seed, coded=True, qk_gain=10.0):
     from safetensors.torch import load_file, save_file
     from sonicboom_amd.weights import write_random_model
     folder = str(tmp_path_factory.mktemp(f"fitatar_{name}"))
     write_random_model(folder, json.loads(json.dumps(cfg)), seed=seed, dtype="bfloat16", device=None)
     path = os.path.join(folder, "model.safetensors")
-    w = sharpen(cfg, {k: v.float().numpy() for k, v in load_file(path).items()}, coded)
+    w = sharpen(cfg, {k: v.float().numpy() for k, v in load_file(path).items()}, coded, qk_gain)
     save_file({k: torch.from_numpy(np.asarray(v, dtype=np.float32)).to(BF16).contiguous() for k, v in w.items()}, path,
               metadata={"format": "pt"})
     plain = {k: v.float().numpy().astype(np.float64) for k, v in load_file(path).items()}
@@ -402,6 +402,68 @@ def test_command_line_and_trace_replay(folders, tmp_path):
         close(read(2), wa[71:72], dtype, "replay, a step where one request wants nothing")
         close(read(3), np.stack([wa[72], wb[11]]), dtype, "replay, last step of the short request")
         close(read(4), wa[74:75], dtype, "replay, two more tokens alone")
+
+
+def drawn_configuration(seed):
+    """A configuration from a seed: two to five layers in any order of kinds (a latent layer may read an earlier
+    one's rows), head counts with one, several and as many kv heads as heads, sizes with and without factors of 8
+    and 16, partly rotated heads, rotations with and without stretched frequencies, every kind of feed-forward and
+    none, routers with and without groups and with and without the expert that every row takes."""
+    rng = np.random.default_rng(1000 + seed)
+    pick = lambda *v: v[int(rng.integers(len(v)))]
+    width = pick(48, 64, 72, 100, 128, 192)
+    layers, latents = [], {}
+    for i in range(int(rng.integers(2, 6))):
+        kind = pick("dense", "moe", "moe", None)
+        if kind == "dense":
+            mlp = {"kind": "dense", "ff": pick(40, 64, 100, 136)}
+        elif kind == "moe":
+            experts = pick(2, 3, 4, 6, 8, 12)
+            count = pick(*[g for g in (1, 2, 3, 4, 6) if experts % g == 0])
+            keep = int(rng.integers(1, count + 1))
+            top = int(rng.integers(1, keep * (experts // count) + 1))
+            mlp = moe(experts, top, pick(8, 20, 32, 48), groups=None if count == 1 and rng.random() < 0.5 else (count, keep),
+                      shared=pick(None, 24, 64))
+        else:
+            mlp = None
+        if rng.random() < 0.5:
+            heads = pick(1, 2, 3, 4, 6, 8)
+            kv_heads = pick(*[g for g in (1, 2, 3, 4, 6, 8) if heads % g == 0])
+            dim = pick(8, 16, 24, 32, 40, 64, 128)
+            layers.append(att(heads, kv_heads, dim, pick(8, 16, 24, 32, 48, 64), float(rng.uniform(0.5, 1.5)) / np.sqrt(dim), mlp,
+                              base=pick(100.0, 1e4, 1e6), rot_dims=pick(dim, dim // 2, 2, 0), factor=pick(None, 2.0, 7.5)))
+            continue
+        src = pick(None, *latents) if latents else None
+        if src is None:
+            rot_dim, rank = pick(2, 4, 8, 16, 32), pick(16, 24, 32, 64, 128)
+            base, scaling = pick(300.0, 1e4, 1e6), pick(None, (2.0, 512, 32.0, 1.0), (6.0, 40, 8.0, 0.5))
+            latents[i] = (rot_dim, rank, base, scaling)
+        else:
+            rot_dim, rank, base, scaling = latents[src]
+        dim = pick(8, 16, 24, 32, 64)
+        layers.append(lat(pick(1, 2, 3, 4, 5, 16), dim, rot_dim, pick(8, 16, 24, 32, 64), rank, pick(8, 12, 48, 80),
+                          float(rng.uniform(0.5, 1.5)) / np.sqrt(dim + rot_dim), mlp, base=base, scaling=scaling, kv_from=src))
+    return config(pick(97, 128, 300, 512), width, layers, eps=pick(1e-6, 1e-5, 1e-3), embed_scale=pick(0.5, 1.0, 6.0),
+                  softcap=pick(0.0, 10.0, 25.0))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_configurations_drawn_from_seeds(tmp_path_factory, seed):
+    cfg = drawn_configuration(seed)
+    # (scores less spread than in the three models above: a drawn shape may have one head of few numbers, where a
+    # spread of ten units makes near ties between keys that bfloat16 rounding decides)
+    folder, plain = make_folder(tmp_path_factory, f"drawn{seed}", cfg, 500 + seed, qk_gain=5.0)
+    rng = np.random.default_rng(seed)
+    reqs = [[int(t) for t in rng.integers(0, cfg["vocab"], size=n)] for n in (150, 9, 71)]
+    want = [P.forward(cfg, plain, r) for r in reqs]
+    for dtype in DTYPES:
+        eng = engine_for(folder, dtype, max_tokens=64 * 8)
+        close(run_whole(eng, reqs[0]), want[0], dtype, f"seed {seed} whole")
+        close(run_tail_one_by_one(eng, reqs[0], tail=40), want[0], dtype, f"seed {seed} tail one by one")
+        for r, w, g in zip(reqs, want, run_batch(eng, reqs, [100, 3, 70])):
+            close(g, w, dtype, f"seed {seed} batch, request of {len(r)}")
+        assert eng.cache.held_pages() == 0 and not eng.cache.live_slots
+        _ENGINES.clear()
 
 
 # ---- mechanisms alone ---------------------------------------------------------------------------
