@@ -738,7 +738,7 @@ def fitatar_sizes(width, vocab=32768, experts=8, top=2):
             layers.append({"type": "latent_attention", "mixer": dict(lat, kv_from=0), "mlp": routed})
         else:
             layers.append({"type": "attention", "mixer": dict(att), "mlp": routed})
-    return {"architecture": "Fitatar", "vocab": vocab, "width": width, "embedding": {"scale": 0.5}, "logit_softcap": 30.0,
+    return {"architecture": "Fitatar", "vocab": vocab, "width": width, "embedding": {"scale": 2.0}, "logit_softcap": 30.0,
             "norm": {"eps": 1e-6}, "layers": layers}
 
 

@@ -166,7 +166,7 @@ def test_configuration_errors_name_the_key(edit, message):
 
 def test_the_package_stretches_frequencies_like_the_plain_implementation():
     from sonicboom_amd.parts.position import stretched_frequencies
-    for dims, base, sc in [(32, 1e6, (2.0, 512, 32.0, 1.0)), (8, 100.0, (5.0, 40, 4.0, 0.5)), (64, 1e4, (40.0, 4096, 32.0, 1.0)),
+    for dims, base, sc in [(32, 5e5, (2.5, 640, 24.0, 1.0)), (8, 100.0, (5.0, 40, 4.0, 0.5)), (64, 1e4, (40.0, 4096, 32.0, 1.0)),
                            (4, 50.0, (1.5, 8, 2.0, 1.0))]:
         rot = {"dims": dims, "base": base, "scaling": {"factor": sc[0], "original": sc[1], "fast": sc[2], "slow": sc[3]}}
         f, m = P.frequencies(rot, "yarn")

@@ -436,7 +436,7 @@ def drawn_configuration(seed):
         src = pick(None, *latents) if latents else None
         if src is None:
             rot_dim, rank = pick(2, 4, 8, 16, 32), pick(16, 24, 32, 64, 128)
-            base, scaling = pick(300.0, 1e4, 1e6), pick(None, (2.0, 512, 32.0, 1.0), (6.0, 40, 8.0, 0.5))
+            base, scaling = pick(300.0, 1e4, 1e6), pick(None, (2.5, 384, 24.0, 1.0), (6.0, 40, 8.0, 0.5))
             latents[i] = (rot_dim, rank, base, scaling)
         else:
             rot_dim, rank, base, scaling = latents[src]
@@ -543,7 +543,7 @@ def test_dense_feed_forward_with_biases(dtype, rows, width, inner):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("rows", [1, 3, 70, 300])
 @pytest.mark.parametrize("experts, top, inner, shared, groups", [
-    (4, 1, 48, 0, None), (6, 3, 32, 64, (3, 2)), (3, 3, 20, 36, None), (9, 2, 136, 16, (3, 1)), (8, 4, 64, 96, (4, 3))])
+    (4, 1, 48, 0, None), (6, 3, 32, 64, (3, 2)), (3, 3, 20, 36, None), (9, 2, 136, 16, (3, 1)), (8, 3, 56, 80, (4, 2))])
 def test_routed_experts_alone(dtype, rows, experts, top, inner, shared, groups):
     """The router's scores over all experts, the choice within the best groups, the experts' products (grouped by
     expert on the matrix cores in bfloat16 when the sizes allow, else a thread an output), the shared expert and
@@ -681,7 +681,7 @@ def latent_mixer(dtype, heads, dim, rot_dim, vdim, rank, q_rank, scale, scaling,
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads, dim, rot_dim, vdim, rank, q_rank, scaling", [
     (4, 32, 16, 48, 64, 40, (4.0, 64, 16.0, 1.0)), (1, 10, 6, 14, 20, 9, None), (3, 24, 16, 8, 48, 16, (1.5, 32, 4.0, 2.0)),
-    (16, 16, 8, 16, 32, 24, (16.0, 128, 32.0, 1.0)), (2, 64, 32, 64, 128, 80, (2.0, 512, 32.0, 1.0))])
+    (16, 16, 8, 16, 32, 24, (16.0, 128, 32.0, 1.0)), (2, 48, 32, 80, 96, 56, (3.0, 256, 16.0, 1.0))])
 def test_latent_attention_alone(dtype, heads, dim, rot_dim, vdim, rank, q_rank, scaling):
     """Queries through their own normed latent, the cached latent row with the shared rotated part, stretched
     frequencies with their magnitude, a gate a head: whole, in portions and token by token; and a second mixer
